@@ -85,8 +85,11 @@ class LLMEngine:
         self.graph_s = executor.capture()
         self.num_blocks = nb
         runner = executor.runner
+        # cached prefix pages hold keys and values only: a model with recurrent layers has
+        # to run the prefix itself to rebuild its state, so it takes no prefix hits
         self.bm = BlockManager(nb, cfg.block_size, cfg.max_num_seqs, runner.max_blocks,
-                               enable_prefix_caching=cfg.enable_prefix_caching)
+                               enable_prefix_caching=cfg.enable_prefix_caching
+                               and not self.mcfg.has_recurrent_state)
         # PP > 1: one micro-batch per stage in flight (engine/scheduler.VirtualSchedulers)
         self.pp_depth = int(getattr(executor, "pipeline_depth", 1))
         if self.pp_depth > 1:

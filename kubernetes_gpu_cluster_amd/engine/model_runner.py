@@ -90,6 +90,7 @@ class Layout:
         self.ws, o = o, o + self.Wmax
         self.wm, o = o, o + self.Wmax
         self.topk, o = o, o + self.Smax
+        self.sslot, o = o, o + self.Smax      # step sequence -> state slot (recurrent layers)
         self.n32 = o
         self.temp, self.topp = 0, self.Smax
         self.nf = 2 * self.Smax
@@ -138,7 +139,13 @@ class ModelRunner:
                                               mcfg.rope_scaling).to(device)
         self.kv = None
         self.kv_caches: list = []
+        self.states: list = []      # per recurrent layer: fp32 state tensors, one slot per sequence
         self.workspace = None
+        # hybrid decoders: per-layer cache / state shapes and step buffers come from the model
+        self.cache_layout = getattr(model, "cache_layout", lambda: None)()
+        self.state_layout = getattr(model, "state_layout", lambda: [])()
+        if hasattr(model, "prepare"):
+            model.prepare(rope_len + 1, max_tokens, device)
         self.graphs: dict[int, tuple] = {}
         self.graph_pool = None
         self.sample_out = torch.zeros(max_num_seqs, dtype=torch.int64, device=device)
@@ -185,6 +192,9 @@ class ModelRunner:
     # ------------------------------------------------------------------ KV cache
     def kv_bytes_per_block(self) -> int:
         m = self.model
+        if self.cache_layout is not None:
+            el = torch.tensor([], dtype=self.kv_dtype).element_size()
+            return max(1, sum(g * (dk + dv) for g, dk, dv in self.cache_layout) * self.bs * el)
         return (2 * m.num_local_layers * m.local_kv_heads() * self.mcfg.head_dim * self.bs *
                 torch.tensor([], dtype=self.kv_dtype).element_size())
 
@@ -209,11 +219,12 @@ class ModelRunner:
         peak = torch.cuda.max_memory_allocated() - base
         self.kv = None
         self.kv_caches = []
+        self.states = []
         torch.cuda.empty_cache()
         free, total = torch.cuda.mem_get_info()
         used_now = total - free
         reserve_graphs = 2 << 30 if self.use_graphs else 0
-        budget = total * gpu_mem_util - used_now - peak - reserve_graphs
+        budget = total * gpu_mem_util - used_now - peak - reserve_graphs - self.state_bytes()
         nb = int(budget // self.kv_bytes_per_block())
         return max(nb, 2)
 
@@ -224,6 +235,7 @@ class ModelRunner:
         self.graph_pool = None
         self.kv = None
         self.kv_caches = []
+        self.states = []
         self.workspace = None
         if self.is_gpu:
             import gc
@@ -231,8 +243,32 @@ class ModelRunner:
             torch.cuda.synchronize()
             torch.cuda.empty_cache()
 
+    def state_bytes(self) -> int:
+        """Bytes of the recurrent layers' per-sequence state (one slot per sequence)."""
+        return sum(4 * self.max_num_seqs * (h * d * dv + h * d + h)
+                   for h, d, dv in self.state_layout)
+
+    def _init_states(self) -> None:
+        """Per recurrent layer (S [slots, H, d, dv], n [slots, H, d], m [slots, H]) in fp32.
+        Zero-filled once; a sequence's first token restarts its slot from zero by itself."""
+        n = self.max_num_seqs
+        self.states = [(torch.zeros(n, h, d, dv, dtype=torch.float32, device=self.device),
+                        torch.zeros(n, h, d, dtype=torch.float32, device=self.device),
+                        torch.zeros(n, h, dtype=torch.float32, device=self.device))
+                       for h, d, dv in self.state_layout]
+
     def init_kv_cache(self, num_blocks: int) -> None:
         m = self.model
+        self._init_states()
+        if self.cache_layout is not None:
+            # plain row-major pages per attention layer: k [nb, G, bs, dk], v [nb, G, bs, dv]
+            self.kv = [(torch.zeros(num_blocks, g, self.bs, dk, dtype=self.kv_dtype,
+                                    device=self.device),
+                        torch.zeros(num_blocks, g, self.bs, dv, dtype=self.kv_dtype,
+                                    device=self.device)) for g, dk, dv in self.cache_layout]
+            self.kv_caches = list(self.kv)
+            self.num_blocks = num_blocks
+            return
         L, nkv, d = m.num_local_layers, m.local_kv_heads(), self.mcfg.head_dim
         # zero-init: stale slots of partially filled blocks must hold finite values
         self.kv = torch.zeros(L, 2, num_blocks, nkv, self.bs, d, dtype=self.kv_dtype,
@@ -276,6 +312,7 @@ class ModelRunner:
         i32[L.ws:L.ws + len(ws)] = ws
         i32[L.wm:L.wm + len(wm)] = wm
         i64[L.lidx:L.lidx + P] = qsl[1:] - 1
+        i32[L.sslot:L.sslot + P] = -1          # no state slot: recurrent layers write nothing
         self.hf.numpy()[: 2 * self.L.Smax] = 1.0
         i64[L.sslots:L.sslots + P] = 0
         # (no TP overlap split in the profiling step: every rank runs it from its own
@@ -307,6 +344,7 @@ class ModelRunner:
             row = table[seq.slot]
             i64[L.slots + off:L.slots + off + n] = row[pos // bs].astype(np.int64) * bs + pos % bs
             i32[L.pbt + i * mb:L.pbt + (i + 1) * mb] = row
+            i32[L.sslot + i] = seq.slot
             qlens.append(n)
             slens.append(a + n)
             off += n
@@ -343,7 +381,9 @@ class ModelRunner:
             dbt = i32[L.dbt:L.dbt + n * mb].reshape(n, mb)
             dbt[:D] = table[slots]
             i32[L.ctx:L.ctx + D] = pos + 1
+            i32[L.sslot + P:L.sslot + P + D] = slots
             if n > D:   # graph padding rows
+                i32[L.sslot + P + D:L.sslot + P + n] = -1
                 i64[L.ids + Tp + D:L.ids + Tp + n] = 0
                 i64[L.pos + Tp + D:L.pos + Tp + n] = 0
                 i64[L.slots + Tp + D:L.slots + Tp + n] = -1
@@ -408,6 +448,8 @@ class ModelRunner:
         d32 = self.d32
         m = AttnMetadata(slot_mapping=self.d64[L.slots:L.slots + T], num_prefill_tokens=Tp,
                          num_prefills=P, num_decodes=D)
+        if self.state_layout:
+            m.state_slots = d32[L.sslot:L.sslot + P + D]
         if P:
             m.prefill_block_tables = d32[L.pbt:L.pbt + P * mb].view(P, mb)
             m.query_start_loc = d32[L.qsl:L.qsl + P + 1]
@@ -417,9 +459,10 @@ class ModelRunner:
         if D:
             m.decode_block_tables = d32[L.dbt:L.dbt + D * mb].view(D, mb)
             m.decode_ctx_lens = d32[L.ctx:L.ctx + D]
-            m.decode_workspace = self.workspace
-            nkv = self.model.local_kv_heads()
-            m.decode_grid_z = z if z is not None else ops.decode_grid_z(D, nkv, max_ctx)
+            if self.cache_layout is None:
+                m.decode_workspace = self.workspace
+                nkv = self.model.local_kv_heads()
+                m.decode_grid_z = z if z is not None else ops.decode_grid_z(D, nkv, max_ctx)
         elif P and split:
             m.split = self._split_prefill(Tp, P)
         return m
@@ -508,7 +551,8 @@ class ModelRunner:
 
     def _forward(self, T, meta: AttnMetadata, hidden_in=None):
         L = self.L
-        ctx = ForwardContext(meta, self.kv_caches, self.cos_sin, *self.kv_scales)
+        ctx = ForwardContext(meta, self.kv_caches, self.cos_sin, *self.kv_scales,
+                             states=self.states)
         ids = self.d64[L.ids:L.ids + T]
         pos = self.d64[L.pos:L.pos + T]
         if self.model.first:
@@ -517,7 +561,18 @@ class ModelRunner:
         return self.model(None, pos, ctx, hidden=h, residual=r)
 
     @torch.inference_mode()
-    def run(self, plan: StepPlan) -> Optional[torch.Tensor]:
+    def run_logits(self, plan: StepPlan, rows: list[int]) -> torch.Tensor:
+        """Execute one step and return the fp32 logits [len(rows), vocab] of the given
+        token rows of the step instead of sampling: teacher-forced replay and scoring
+        (engine/replay.py).  Cache, state and graph use are those of ``run``."""
+        idx = torch.tensor(rows, dtype=torch.int64)
+        if self.is_gpu:
+            idx = idx.pin_memory().to(self.device, non_blocking=True)
+        return self.run(plan, logit_rows=idx)
+
+    @torch.inference_mode()
+    def run(self, plan: StepPlan, logit_rows: Optional[torch.Tensor] = None
+            ) -> Optional[torch.Tensor]:
         """Execute one step on this rank.  Returns sampled ids [S] (last PP stage)."""
         if ops.DEBUG and self.is_gpu:
             ops.debug_check()           # the previous step's kernels (bounds-checking build)
@@ -547,7 +602,7 @@ class ModelRunner:
             self.stats["graph_steps"] += 1
             if not self.model.last:
                 return None
-            logits = logits[: plan.S]
+            logits = logits[: plan.S] if logit_rows is None else logits.index_select(0, logit_rows)
             T = plan.B
         else:
             T = plan.T if not plan.B else plan.B
@@ -558,17 +613,19 @@ class ModelRunner:
             if not self.model.last:
                 comm.pp_send(list(out))
                 return None
-            idx = self.d64[L.lidx:L.lidx + plan.S]
+            idx = self.d64[L.lidx:L.lidx + plan.S] if logit_rows is None else logit_rows
             logits = self.model.compute_logits(out.index_select(0, idx), gather=not self.vp)
         if ps.tp_size > 1:
             self._count_tp_bytes(plan, T)
         if self.vp:                 # logits are this rank's vocabulary shard
-            if plan.vp:
+            if plan.vp and logit_rows is None:
                 res = self._sample_vp(logits, plan)
                 self.last_tok.index_copy_(0, self.d64[L.sslots:L.sslots + plan.S], res)
                 self._last_lp = None
                 return res
             logits = comm.tp_all_gather(logits, -1)[:, : self.mcfg.vocab_size]
+        if logit_rows is not None:
+            return logits.float()
         pre_lp = None
         if plan.proc and self.model.last:
             if plan.lp:       # logprobs report the raw distribution, before processing
@@ -698,7 +755,7 @@ class ModelRunner:
         """Capture decode forward + LM head for each batch bucket (largest first,
         sharing one memory pool).  Returns seconds spent."""
         self.buckets = graph_buckets(self.graph_max_bs)
-        if self.is_gpu:
+        if self.is_gpu and self.dtype != torch.float32:
             # K9: per decode bucket and weight shape, hipBLASLt or the skinny GEMM --
             # whichever measured faster on this model's weights (ops/gemm.py)
             from ..ops import gemm
@@ -732,6 +789,7 @@ class ModelRunner:
         self.h64.zero_()
         self.h32.zero_()
         self.h64[L.slots:L.slots + self.graph_max_bs] = -1
+        self.h32[L.sslot:L.sslot + self.graph_max_bs] = -1
         self.h64[L.lidx:L.lidx + self.graph_max_bs] = torch.arange(self.graph_max_bs)
         self.d64.copy_(self.h64)
         self.d32.copy_(self.h32)

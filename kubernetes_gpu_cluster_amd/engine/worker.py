@@ -343,6 +343,10 @@ class LocalExecutor:
             sh.raise_if_failed(slot)
         return res
 
+    def execute_logits(self, plan: StepPlan, rows: list) -> torch.Tensor:
+        """Run the step and return the fp32 logits of its token rows ``rows`` (no sampling)."""
+        return self.worker.runner.run_logits(plan, rows)
+
     def execute_async(self, plan: StepPlan) -> "TokenFuture":
         out = self.worker.run(plan)
         sh = self.worker.sampler_health

@@ -17,6 +17,7 @@ from typing import Iterable, Iterator, Optional
 import torch
 
 from .configs import PRESETS, ModelConfig, resolve_model
+from .dilavik import DilavikForCausalLM
 from .llama import LlamaForCausalLM
 from .opt import OPTForCausalLM
 
@@ -24,6 +25,8 @@ from .opt import OPTForCausalLM
 def build_model(cfg: ModelConfig, dtype=torch.bfloat16, device=None):
     if cfg.arch == "opt":
         return OPTForCausalLM(cfg, dtype, device)
+    if cfg.arch == "dilavik":
+        return DilavikForCausalLM(cfg, dtype, device)
     return LlamaForCausalLM(cfg, dtype, device)
 
 
@@ -35,7 +38,11 @@ def _seed_for(name: str, base: int) -> int:
 @torch.no_grad()
 def random_init(model: torch.nn.Module, seed: int = 0, std: float = 0.02) -> None:
     """Deterministic per-parameter random init, generated on the parameter's device
-    (fast for 70B-class shards).  Norm weights stay at 1; biases small."""
+    (fast for 70B-class shards).  Norm weights stay at 1; biases small.  A model with
+    parameters of other kinds initialises them itself (``init_random``)."""
+    if hasattr(model, "init_random"):
+        model.init_random(seed, std)
+        return
     for name, p in model.named_parameters():
         if "norm" in name and name.endswith("weight"):
             p.fill_(1.0)

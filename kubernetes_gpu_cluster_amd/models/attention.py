@@ -37,6 +37,9 @@ class AttnMetadata:
     # prefill-only TP step split into two token halves for comm/compute overlap:
     # (a, meta of tokens [0, a), meta of tokens [a, T)) -- engine/model_runner.py
     split: Optional[tuple] = None
+    # recurrent layers: the state slot of every step sequence (prefill chunks first, then
+    # decode rows; < 0: a graph padding row) -- int32 [P + D]
+    state_slots: Optional[torch.Tensor] = None
 
 
 @dataclasses.dataclass
@@ -46,6 +49,8 @@ class ForwardContext:
     cos_sin: Optional[torch.Tensor] = None
     k_scale: float = 1.0                               # fp8 KV: cache holds fp8(x / scale)
     v_scale: float = 1.0
+    # per recurrent layer: its state tensors, one slot per running sequence
+    states: Optional[list] = None
 
 
 class PagedAttention(nn.Module):
@@ -77,3 +82,49 @@ class PagedAttention(nn.Module):
             if o.data_ptr() != dst.data_ptr():
                 dst.copy_(o)
         return out.view(q.shape[0], self.nq * self.d)
+
+
+class WindowedAttention(nn.Module):
+    """Attention mixer of the hybrid decoders: GQA with separate query/key and value
+    sizes, rotary on the first ``rot_dims`` dimensions of a head, a sliding window that
+    keeps the first tokens visible, softmax in fp32, and a per-head sigmoid output gate
+    computed from the mixer's input.  Keys and values live in a plain-layout paged cache
+    (k [nb, G, bs, dim], v [nb, G, bs, vdim]) indexed by the engine's block tables, so
+    chunked prefill and decode rows of one step run through the same kernels."""
+
+    def __init__(self, hidden: int, spec, cache_idx: int, dtype, device):
+        super().__init__()
+        from ..parallel.layers import ReplicatedLinear
+        self.spec, self.cache_idx = spec, cache_idx
+        H, G, dk, dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
+        assert H % G == 0, "query heads must be a multiple of key/value heads"
+        assert spec.rot_dims % 2 == 0 and spec.rot_dims <= dk
+        self.qkv_proj = ReplicatedLinear(hidden, H * dk + G * dk + G * dv, dtype=dtype,
+                                         device=device)
+        self.o_proj = ReplicatedLinear(H * dv, hidden, dtype=dtype, device=device)
+        self.gate = (nn.Parameter(torch.zeros(H, hidden, dtype=dtype, device=device),
+                                  requires_grad=False) if spec.head_gate else None)
+        self.scale = spec.dim ** -0.5 if spec.scale is None else spec.scale
+        self.rope = None            # [max_pos, rot_dims] fp32, set by prepare()
+
+    def prepare(self, tables: dict, max_pos: int, device) -> None:
+        sp = self.spec
+        if not sp.rot_dims:
+            return
+        key = (sp.rot_dims, sp.rot_base)
+        if key not in tables:
+            tables[key] = ops.ref.rope_table(sp.rot_dims, max_pos, sp.rot_base).to(device)
+        self.rope = tables[key]
+
+    def forward(self, h: torch.Tensor, positions: torch.Tensor, ctx: ForwardContext):
+        sp = self.spec
+        kc, vc = ctx.kv_caches[self.cache_idx]
+        qkv = self.qkv_proj(h)
+        gate = (ops.gate_proj(h, self.gate, None, ops.GATE_SIGMOID)
+                if self.gate is not None else None)
+        q = ops.rope_kv_store(qkv, positions, self.rope, kc, vc, ctx.attn.slot_mapping,
+                              sp.heads, sp.kv_heads, sp.dim, sp.vdim)
+        w = sp.window
+        o = ops.window_attention(q, kc, vc, positions, ctx.attn, self.scale,
+                                 w.size if w else 0, w.keep_first if w else 0, gate)
+        return self.o_proj(o)

@@ -18,6 +18,38 @@ import os
 from typing import Optional
 
 
+@dataclasses.dataclass(frozen=True)
+class WindowSpec:
+    """Sliding-window visibility with kept first tokens: query i sees key j when
+    j <= i and (i - j < size or j < keep_first)."""
+    size: int
+    keep_first: int = 0
+
+
+@dataclasses.dataclass(frozen=True)
+class MixerSpec:
+    """One layer of a hybrid decoder: its token mixer and (optional) feed-forward.
+
+    kind "attention": softmax attention over a paged KV cache (GQA, per-head query/key
+    size ``dim`` and value size ``vdim``, rotary on the first ``rot_dims`` dimensions,
+    an optional window, an optional per-head sigmoid output gate).
+    kind "mlstm": matrix-memory recurrence (one [dim, vdim] fp32 state per head and
+    sequence, exponential gating capped at ``gate_cap``)."""
+    kind: str
+    heads: int
+    dim: int
+    vdim: int
+    kv_heads: int = 0
+    scale: Optional[float] = None
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    window: Optional[WindowSpec] = None
+    head_gate: bool = False
+    gate_cap: float = 0.0
+    ff: int = 0                  # 0: the layer has no feed-forward sublayer
+    ff_kind: str = "dense"
+
+
 @dataclasses.dataclass
 class ModelConfig:
     name: str
@@ -48,6 +80,11 @@ class ModelConfig:
     top_k_experts: int = 0
     bos_token_id: int = 1
     eos_token_id: int = 2
+    # hybrid decoders (arch "dilavik"): one MixerSpec per layer, a grouped RMSNorm, a
+    # scaled embedding and learned depth-weighted averaging of the layer results
+    layer_specs: Optional[tuple] = None
+    norm_groups: int = 1
+    embed_scale: float = 1.0
 
     @property
     def q_size(self) -> int:
@@ -61,8 +98,23 @@ class ModelConfig:
     def is_moe(self) -> bool:
         return self.num_experts > 0
 
+    @property
+    def has_recurrent_state(self) -> bool:
+        """A layer carries per-sequence state outside the paged KV cache: cached prefix
+        blocks cannot stand in for computing the prefix."""
+        return any(sp.kind != "attention" for sp in (self.layer_specs or ()))
+
     def num_params(self) -> int:
         h, i, L = self.hidden_size, self.intermediate_size, self.num_layers
+        if self.layer_specs:
+            n = 2 * self.vocab_size * h
+            for sp in self.layer_specs:
+                if sp.kind == "attention":
+                    n += h * (sp.heads * sp.dim + sp.kv_heads * (sp.dim + sp.vdim) + sp.heads)
+                else:
+                    n += h * (2 * sp.heads * sp.dim + 2 * sp.heads * sp.vdim + 2 * sp.heads)
+                n += sp.heads * sp.vdim * h + 2 * h * sp.ff
+            return n
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         if self.act == "silu":
             mlp = 3 * h * i
@@ -74,6 +126,9 @@ class ModelConfig:
         return L * (attn + mlp) + emb
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        if self.layer_specs:
+            return sum(sp.kv_heads * (sp.dim + sp.vdim) * dtype_bytes
+                       for sp in self.layer_specs if sp.kind == "attention")
         return 2 * self.num_layers * self.num_kv_heads * self.head_dim * dtype_bytes
 
     def shrink(self, **kw) -> "ModelConfig":
@@ -158,8 +213,48 @@ _ALIASES = {
 }
 
 
+def _mixer_spec(entry: dict) -> MixerSpec:
+    """One entry of a hybrid config's ``layers`` list -> MixerSpec."""
+    kind, m, mlp = entry["type"], entry["mixer"], entry.get("mlp")
+    ff = int(mlp["ff"]) if mlp else 0
+    ff_kind = mlp.get("kind", "dense") if mlp else "dense"
+    if ff and ff_kind != "dense":
+        raise ValueError(f"unsupported feed-forward kind {ff_kind!r}")
+    if kind == "attention":
+        rot, mask = m.get("rot"), m.get("mask")
+        return MixerSpec("attention", int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                         kv_heads=int(m.get("kv_heads", m["heads"])), scale=float(m["scale"]),
+                         rot_dims=int(rot["dims"]) if rot else 0,
+                         rot_base=float(rot["base"]) if rot else 10000.0,
+                         window=WindowSpec(int(mask["size"]), int(mask.get("keep_first", 0)))
+                         if mask else None,
+                         head_gate=True, ff=ff, ff_kind=ff_kind)
+    if kind == "mlstm":
+        return MixerSpec("mlstm", int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                         gate_cap=float(m["gate_cap"]), ff=ff, ff_kind=ff_kind)
+    raise ValueError(f"unknown mixer type {kind!r}")
+
+
+def dilavik_config(d: dict, name: str) -> ModelConfig:
+    """A Dilavik config.json (``architecture``, ``width``, ``vocab``, ``layers``, ``norm``,
+    ``embedding``) -> ModelConfig.  The flat attention fields describe the first attention
+    layer (reporting only); the engine sizes caches and state from ``layer_specs``."""
+    specs = tuple(_mixer_spec(e) for e in d["layers"])
+    att = next((sp for sp in specs if sp.kind == "attention"), specs[0])
+    return ModelConfig(
+        name, "dilavik", len(specs), int(d["width"]), att.heads, att.kv_heads or att.heads,
+        att.dim, max((sp.ff for sp in specs), default=0), int(d["vocab"]),
+        max_position=int(d.get("max_position", 8192)), rope_theta=att.rot_base,
+        rms_eps=float(d["norm"]["eps"]), layer_specs=specs,
+        norm_groups=int(d["norm"].get("groups", 1)),
+        embed_scale=float(d.get("embedding", {}).get("scale", 1.0)),
+        bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)))
+
+
 def _from_hf_config(d: dict, name: str) -> ModelConfig:
     """Map an HF config.json dict onto ModelConfig."""
+    if d.get("architecture") == "Dilavik":
+        return dilavik_config(d, name)
     mt = d.get("model_type", "llama")
     if mt == "opt":
         h = d["hidden_size"]

@@ -1,0 +1,59 @@
+"""Recurrent token mixers: layers whose memory is a fixed-size per-sequence state
+instead of a growing KV cache.
+
+The engine gives every running sequence a state slot (the sequence's block-table row
+index, ``engine/block_manager.py``); a layer's state tensors hold one entry per slot
+(``ModelRunner.init_kv_cache``), and a step's ``AttnMetadata.state_slots`` names the slot
+of each step sequence.  A sequence's first token (position 0) starts from the zero state,
+so a slot is reused, and a preempted sequence recomputed, without any clearing pass.
+State is fp32 and carried from step to step: chunked prefill and decode rows run through
+the same scan kernel.
+"""
+from __future__ import annotations
+
+import torch
+import torch.nn as nn
+
+from .. import ops
+from ..parallel.layers import ReplicatedLinear
+from .attention import ForwardContext
+
+
+class MLSTMMixer(nn.Module):
+    """Matrix-memory LSTM (the mLSTM of xLSTM): per head a [dim, vdim] memory S, a
+    normaliser n and a running log-scale m (starting at 0).  With capped log gates
+    i = cap tanh((W_i h + b_i) / cap) and f = logsigmoid(cap tanh((W_f h + b_f) / cap)):
+        m' = max(f + m, i);  S' = e^(f + m - m') S + e^(i - m') k v^T;  n' likewise with k
+        o  = S'^T q / (max(|n'.q|, e^(-m')) + 1e-6),   q scaled by dim^-1/2
+    then each head's o over its RMS, times a learned weight, times sigmoid(W_g h), and the
+    output projection.  The gates, the scan and the head norm run in fp32."""
+
+    def __init__(self, hidden: int, spec, state_idx: int, eps: float, dtype, device):
+        super().__init__()
+        self.spec, self.state_idx, self.eps = spec, state_idx, eps
+        H, d, dv = spec.heads, spec.dim, spec.vdim
+        # q | k | v | output-gate pre-activation, one GEMM
+        self.qkvg_proj = ReplicatedLinear(hidden, 2 * H * d + 2 * H * dv, dtype=dtype,
+                                          device=device)
+        self.o_proj = ReplicatedLinear(H * dv, hidden, dtype=dtype, device=device)
+        # log input gates | log forget gates
+        self.if_weight = nn.Parameter(torch.zeros(2 * H, hidden, dtype=dtype, device=device),
+                                      requires_grad=False)
+        self.if_bias = nn.Parameter(torch.zeros(2 * H, dtype=torch.float32, device=device),
+                                    requires_grad=False)
+        self.norm_weight = nn.Parameter(torch.ones(H * dv, dtype=torch.float32, device=device),
+                                        requires_grad=False)
+
+    def state_shapes(self) -> tuple:
+        sp = self.spec
+        return (sp.heads, sp.dim, sp.vdim)
+
+    def forward(self, h: torch.Tensor, positions: torch.Tensor, ctx: ForwardContext):
+        sp = self.spec
+        H, d, dv = sp.heads, sp.dim, sp.vdim
+        qkvg = self.qkvg_proj(h)
+        gates = ops.gate_proj(h, self.if_weight, self.if_bias, ops.GATE_CAP_TANH,
+                              ops.GATE_LOGSIG_CAP_TANH, H, sp.gate_cap)
+        o = ops.mlstm_scan(qkvg, gates, ctx.states[self.state_idx], ctx.attn, H, d, dv)
+        g = qkvg[:, 2 * H * d + H * dv:]
+        return self.o_proj(ops.head_norm_gate(o, g, self.norm_weight, H, self.eps, h.dtype))

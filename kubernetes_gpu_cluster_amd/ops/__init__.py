@@ -617,3 +617,152 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
     out = torch.empty(T, H, dtype=x.dtype, device=dev)
     k.moe_combine(out, y, topk_w.contiguous().float())
     return out
+
+
+# ------------------------------------------------------------------ hybrid decoders
+# Grouped RMSNorm over an fp32 residual stream, depth-weighted averaging of the layer
+# results, xIELU, small fp32 gate projections, windowed attention with kept first tokens
+# over a plain-layout paged cache (per-layer query/key and value sizes), and the mLSTM
+# matrix-memory scan over per-sequence state slots.  ``meta`` is the step's AttnMetadata.
+GATE_SIGMOID, GATE_CAP_TANH, GATE_LOGSIG_CAP_TANH = (ref.GATE_SIGMOID, ref.GATE_CAP_TANH,
+                                                     ref.GATE_LOGSIG_CAP_TANH)
+
+
+def group_rms_norm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
+                   out_dtype: torch.dtype, add: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """h = grouped RMSNorm(x) * w in ``out_dtype``; x [T, W] is the fp32 residual stream.
+    ``add`` [T, W]: x += add first, in place (the sublayer's output joins the stream)."""
+    if not _gpu(x):
+        if add is not None:
+            x += add.float()
+        return ref.group_rms_norm(x, w, groups, eps, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _k().residual_group_norm(out, x, add, w, groups, eps)
+    return out
+
+
+def depth_mix_norm(x: torch.Tensor, hist: torch.Tensor, layer: int, y: torch.Tensor,
+                   coef: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """End of layer ``layer`` of a depth-averaged decoder, in one pass over the rows:
+    hist[layer + 1, :T] = x + y (the layer's result); x = sum_j coef[j] * hist[j, :T] over
+    j <= layer + 1 (in place: what the next layer reads); returns grouped RMSNorm(x) * w
+    (the next layer's first norm, or the model's final one).  hist [L + 1, Tcap, W] and x
+    are fp32; coef fp32 [layer + 2]."""
+    T = x.shape[0]
+    if not _gpu(x):
+        hist[layer + 1, :T] = x + y.float()
+        x.copy_(ref.depth_mix(hist, layer + 2, coef, T))
+        return ref.group_rms_norm(x, w, groups, eps, out_dtype)
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _k().depth_mix_norm(out, x, hist, y, coef, w, layer, groups, eps)
+    return out
+
+
+def xielu(z: torch.Tensor, ab: torch.Tensor) -> torch.Tensor:
+    """ab fp32 [2] = (softplus(p), 1/2 + softplus(q)) of the layer's two parameters."""
+    if not _gpu(z):
+        return ref.xielu(z, ab)
+    out = torch.empty_like(z)
+    _k().xielu(out, z, ab)
+    return out
+
+
+def gate_proj(h: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], kind_a: int,
+              kind_b: int = 0, split: Optional[int] = None, cap: float = 1.0) -> torch.Tensor:
+    """fp32 [T, N] gate values act(h . w^T + bias) for a few output rows N (per-head
+    gates): the products accumulate and stay in fp32."""
+    split = w.shape[0] if split is None else split
+    if not _gpu(h):
+        return ref.gate_proj(h, w, bias, kind_a, kind_b, split, cap)
+    out = torch.empty(h.shape[0], w.shape[0], dtype=torch.float32, device=h.device)
+    _k().gate_proj(out, h, w, bias, kind_a, kind_b, split, cap)
+    return out
+
+
+def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, table: Optional[torch.Tensor],
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                  H: int, G: int, dk: int, dv: int) -> torch.Tensor:
+    if not _gpu(qkv):
+        return ref.rope_kv_store(qkv, positions, table, k_cache, v_cache, slot_mapping, H, G,
+                                 dk, dv)
+    q = torch.empty(qkv.shape[0], H, dk, dtype=qkv.dtype, device=qkv.device)
+    _k().rope_kv_store(qkv, positions, table, q, k_cache, v_cache, slot_mapping, H, G, dk, dv)
+    return q
+
+
+def _row_tables(meta, T: int) -> torch.Tensor:
+    """CPU path: the block-table row of every token of the step."""
+    rows = []
+    if meta.num_prefills:
+        qsl = meta.query_start_loc.tolist()
+        for i in range(meta.num_prefills):
+            rows.append(meta.prefill_block_tables[i:i + 1].expand(qsl[i + 1] - qsl[i], -1))
+    if meta.num_decodes:
+        rows.append(meta.decode_block_tables[: meta.num_decodes])
+    return torch.cat(rows, 0)[:T]
+
+
+def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     positions: torch.Tensor, meta, scale: float, window: int, keep_first: int,
+                     gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Prefill chunks and decode rows of one step alike: row t sees the cached keys
+    j <= p with p - j < window or j < keep_first (p = positions[t]; window <= 0: plain
+    causal).  Decode padding rows (context length 0) give zeros."""
+    T, H, _ = q.shape
+    dv = v_cache.shape[3]
+    if not _gpu(q):
+        pos = positions.clone()
+        if meta.num_decodes:
+            tp = meta.num_prefill_tokens
+            pos[tp:tp + meta.num_decodes] = meta.decode_ctx_lens[: meta.num_decodes].long() - 1
+        return ref.window_attention(q, k_cache, v_cache, pos, _row_tables(meta, T), scale,
+                                    window, keep_first, gate)
+    out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    _k().window_attention(out, q, k_cache, v_cache, meta.query_start_loc,
+                          meta.prefill_seq_lens, meta.prefill_block_tables,
+                          meta.decode_ctx_lens, meta.decode_block_tables,
+                          meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens,
+                          scale, window, keep_first, gate)
+    return out
+
+
+def mlstm_scan(qkvg: torch.Tensor, gates: torch.Tensor, state: tuple, meta, H: int, d: int,
+               dv: int) -> torch.Tensor:
+    """fp32 [T, H*dv]: the matrix-memory recurrence over every step sequence's tokens,
+    read from and written back to its state slot (``meta.state_slots``; < 0: a padding
+    row, skipped).  state = (S [slots, H, d, dv], n [slots, H, d], m [slots, H]) fp32."""
+    S, n, m = state
+    T = qkvg.shape[0]
+    P, D, tp = meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens
+    if not _gpu(qkvg):
+        start, ln, pos = [], [], []
+        if P:
+            qsl, sl = meta.query_start_loc.tolist(), meta.prefill_seq_lens.tolist()
+            for i in range(P):
+                start.append(qsl[i])
+                ln.append(qsl[i + 1] - qsl[i])
+                pos.append(sl[i] - ln[-1])
+        if D:
+            ctx = meta.decode_ctx_lens.tolist()
+            for i in range(D):
+                start.append(tp + i)
+                ln.append(1)
+                pos.append(ctx[i] - 1)
+        return ref.mlstm_scan(qkvg, gates, S, n, m, start, ln, pos,
+                              meta.state_slots[: P + D].tolist(), H, d, dv)
+    out = torch.empty(T, H * dv, dtype=torch.float32, device=qkvg.device)
+    _k().mlstm_scan(out, qkvg, gates, S, n, m, meta.query_start_loc, meta.prefill_seq_lens,
+                    meta.decode_ctx_lens, meta.state_slots, P, D, tp, H, d, dv)
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, g: torch.Tensor, w: torch.Tensor, H: int, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """Per-head RMS normalisation of the recurrence output o (fp32 [T, H*dv]), times w,
+    times sigmoid(g) (g: a [T, H*dv] column slice of the merged projection)."""
+    if not _gpu(o):
+        return ref.head_norm_gate(o, g, w, H, eps, out_dtype)
+    out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
+    _k().head_norm_gate(out, o, g, w, H, eps)
+    return out

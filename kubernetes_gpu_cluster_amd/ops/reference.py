@@ -358,3 +358,165 @@ def moe_mlp(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torch.
         y = h @ w2[e].float().t()
         out.index_add_(0, tok, y * topk_w[tok, slot, None].float())
     return out.to(x.dtype)
+
+
+# ---------------------------------------------------------------- hybrid decoders
+# (grouped RMSNorm, depth-weighted averaging, xIELU, small gate projections, windowed
+# attention with kept first tokens over a plain-layout paged cache, mLSTM state scan)
+def group_rms_norm(x: torch.Tensor, w: torch.Tensor, groups: int, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """Each of ``groups`` equal consecutive parts of a row is divided by its own
+    sqrt(mean(part^2) + eps); the whole row is then multiplied by w.  fp32 math."""
+    T, W = x.shape
+    xg = x.float().view(T, groups, W // groups)
+    xg = xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps)
+    return (xg.view(T, W) * w.float()).to(out_dtype)
+
+
+def depth_mix(hist: torch.Tensor, n: int, coef: torch.Tensor, T: int) -> torch.Tensor:
+    """sum_j coef[j] * hist[j, :T] over the first n layer results (fp32)."""
+    return torch.einsum("j,jtw->tw", coef[:n].float(), hist[:n, :T].float())
+
+
+def xielu(z: torch.Tensor, ab: torch.Tensor) -> torch.Tensor:
+    """z > 0: a z^2 + z/2;  z <= 0: b (exp(z) - 1 - z) + z/2, with ab = (a, b) fp32."""
+    zf = z.float()
+    a, b = ab[0], ab[1]
+    return torch.where(zf > 0, a * zf * zf + 0.5 * zf,
+                       b * (torch.expm1(torch.clamp(zf, max=0.0)) - zf) + 0.5 * zf).to(z.dtype)
+
+
+GATE_SIGMOID, GATE_CAP_TANH, GATE_LOGSIG_CAP_TANH = 0, 1, 2
+
+
+def _gate_act(y: torch.Tensor, kind: int, cap: float) -> torch.Tensor:
+    if kind == GATE_SIGMOID:
+        return torch.sigmoid(y)
+    y = cap * torch.tanh(y / cap)
+    return y if kind == GATE_CAP_TANH else torch.nn.functional.logsigmoid(y)
+
+
+def gate_proj(h: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], kind_a: int,
+              kind_b: int, split: int, cap: float) -> torch.Tensor:
+    """fp32 [T, N]: act(h . w^T + bias), rows < split of w with kind_a, the rest kind_b.
+    The dot products accumulate in fp32 and are never rounded to 16 bits."""
+    y = h.float() @ w.float().t()
+    if bias is not None:
+        y = y + bias.float()
+    return torch.cat([_gate_act(y[:, :split], kind_a, cap), _gate_act(y[:, split:], kind_b, cap)],
+                     dim=1)
+
+
+def rope_table(rot_dims: int, max_pos: int, base: float) -> torch.Tensor:
+    """[max_pos, rot_dims] fp32: cos | sin of p * base^(-2i/rot_dims), i < rot_dims/2,
+    with the frequencies, the angles and cos / sin all evaluated in fp32."""
+    f = torch.tensor(base, dtype=torch.float32) ** (
+        -2.0 * torch.arange(rot_dims // 2, dtype=torch.float32) / rot_dims)
+    a = torch.arange(max_pos, dtype=torch.float32)[:, None] * f[None]
+    return torch.cat([a.cos(), a.sin()], dim=-1)
+
+
+def rope_kv_store(qkv: torch.Tensor, positions: torch.Tensor, table: Optional[torch.Tensor],
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                  H: int, G: int, dk: int, dv: int) -> torch.Tensor:
+    """qkv [T, H*dk + G*dk + G*dv] -> rotated q [T, H, dk]; rotated k and v go to the
+    plain-layout paged cache (k_cache [nb, G, bs, dk], v_cache [nb, G, bs, dv]) at
+    ``slot_mapping`` (< 0: no write).  Rotation pairs dim i with i + rot/2 over the first
+    rot = table.shape[1] dims of a head (fp32 math); the rest pass unchanged."""
+    T = qkv.shape[0]
+    q = qkv[:, : H * dk].float().view(T, H, dk)
+    k = qkv[:, H * dk: (H + G) * dk].float().view(T, G, dk)
+    v = qkv[:, (H + G) * dk: (H + G) * dk + G * dv].view(T, G, dv)
+    if table is not None:
+        r = table.shape[1]
+        cs = table[positions.long()]
+        c, s = cs[:, None, : r // 2], cs[:, None, r // 2:]
+
+        def rot(x):
+            a, b = x[..., : r // 2], x[..., r // 2: r]
+            return torch.cat([a * c - b * s, b * c + a * s, x[..., r:]], dim=-1)
+        q, k = rot(q), rot(k)
+    bs = k_cache.shape[2]
+    ok = slot_mapping >= 0
+    sl = slot_mapping[ok].long()
+    k_cache[sl // bs, :, sl % bs] = k[ok].to(k_cache.dtype)
+    v_cache[sl // bs, :, sl % bs] = v[ok].to(v_cache.dtype)
+    return q.to(qkv.dtype)
+
+
+def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     positions: torch.Tensor, row_tables: torch.Tensor, scale: float,
+                     window: int, keep_first: int,
+                     gate: Optional[torch.Tensor]) -> torch.Tensor:
+    """q [T, H, dk] (rotated; the step's k / v already stored) -> [T, H*dv].  Row t at
+    position p = positions[t] attends the cached keys j <= p with p - j < window or
+    j < keep_first (window <= 0: all of them) of the sequence whose block table is
+    row_tables[t]; softmax and the weighted sum in fp32; each head's output times
+    gate[t, head] (fp32) when given."""
+    T, H, dk = q.shape
+    G, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    out = torch.zeros(T, H, dv, dtype=torch.float32)
+    for t in range(T):
+        p = int(positions[t])
+        if p < 0:
+            continue
+        j = torch.arange(p + 1)
+        if window > 0:
+            j = j[(p - j < window) | (j < keep_first)]
+        blk = row_tables[t].long()[j // bs]
+        k = k_cache[blk, :, j % bs].float()           # [n, G, dk]
+        v = v_cache[blk, :, j % bs].float()
+        qt = q[t].float().view(G, H // G, dk)
+        s = torch.einsum("ghd,ngd->ghn", qt, k) * scale
+        pr = torch.softmax(s, dim=-1)
+        out[t] = torch.einsum("ghn,ngv->ghv", pr, v).reshape(H, dv)
+    if gate is not None:
+        out = out * gate.float()[:, :, None]
+    return out.view(T, H * dv).to(q.dtype)
+
+
+def mlstm_scan(qkvg: torch.Tensor, gates: torch.Tensor, S: torch.Tensor, n: torch.Tensor,
+               m: torch.Tensor, seq_start: list, seq_len: list, seq_pos: list, seq_slot: list,
+               H: int, d: int, dv: int) -> torch.Tensor:
+    """The mLSTM recurrence over each step sequence's tokens, from (and back into) its
+    state slot: S [slots, H, d, dv], n [slots, H, d], m [slots, H], all fp32.  A sequence
+    whose first token is at position 0 starts from zero state (m = 0).  qkvg [T, >= 2Hd+Hdv]:
+    q | k | v (| ...); gates [T, 2H] fp32: log input gate | log forget gate.  With
+    m' = max(f + m, i):  S' = exp(f + m - m') S + exp(i - m') k v^T, n' likewise with k;
+    o = S'^T q / (max(|n'.q|, exp(-m')) + 1e-6), q scaled by d^-1/2.  -> fp32 [T, H*dv]."""
+    T = qkvg.shape[0]
+    out = torch.zeros(T, H, dv, dtype=torch.float32)
+    qs = d ** -0.5
+    for a, ln, p0, slot in zip(seq_start, seq_len, seq_pos, seq_slot):
+        if slot < 0:
+            continue
+        if p0 == 0:
+            Sx = torch.zeros(H, d, dv)
+            nx = torch.zeros(H, d)
+            mx = torch.zeros(H)
+        else:
+            Sx, nx, mx = S[slot].clone(), n[slot].clone(), m[slot].clone()
+        for t in range(a, a + ln):
+            q = qkvg[t, : H * d].float().view(H, d) * qs
+            k = qkvg[t, H * d: 2 * H * d].float().view(H, d)
+            v = qkvg[t, 2 * H * d: 2 * H * d + H * dv].float().view(H, dv)
+            ig, fg = gates[t, :H], gates[t, H:]
+            mn = torch.maximum(fg + mx, ig)
+            fa, ia = torch.exp(fg + mx - mn), torch.exp(ig - mn)
+            Sx = fa[:, None, None] * Sx + ia[:, None, None] * k[:, :, None] * v[:, None, :]
+            nx = fa[:, None] * nx + ia[:, None] * k
+            mx = mn
+            den = torch.maximum((nx * q).sum(-1).abs(), torch.exp(-mx)) + 1e-6
+            out[t] = torch.einsum("hdv,hd->hv", Sx, q) / den[:, None]
+        S[slot], n[slot], m[slot] = Sx, nx, mx
+    return out.view(T, H * dv)
+
+
+def head_norm_gate(o: torch.Tensor, g: torch.Tensor, w: torch.Tensor, H: int, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """o fp32 [T, H*dv]: each head divided by its root mean square, times w, times
+    sigmoid(g) (g [T, H*dv], any float dtype); fp32 math -> out_dtype."""
+    T, N = o.shape
+    oh = o.float().view(T, H, N // H)
+    oh = oh * torch.rsqrt(oh.pow(2).mean(-1, keepdim=True) + eps)
+    return (oh.view(T, N) * w.float() * torch.sigmoid(g.float())).to(out_dtype)
