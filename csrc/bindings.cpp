@@ -1213,9 +1213,254 @@ std::vector<int64_t> sample_stamps() {
 int64_t decode_wave_min_pairs() { return kgc::paged_decode_wave_min_pairs(); }
 int64_t prefill_block_m() { return kgc::prefill_block_m(); }
 
+// ---- hybrid decoders ---------------------------------------------------------------
+bool act_dtype(const Tensor& t) {
+  return t.scalar_type() == at::kBFloat16 || t.scalar_type() == at::kHalf ||
+         t.scalar_type() == at::kFloat;
+}
+
+void check_f32(const Tensor& t, const char* name) {
+  TORCH_CHECK(t.is_cuda() && t.scalar_type() == at::kFloat && t.is_contiguous(), "kgc: ", name,
+              " must be a contiguous fp32 GPU tensor");
+}
+
+void residual_group_norm(Tensor out, Tensor x, std::optional<Tensor> y, Tensor w, int64_t groups,
+                         double eps) {
+  check_f32(x, "x");
+  check_f32(w, "w");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+  TORCH_CHECK(x.dim() == 2 && out.is_contiguous() && out.sizes() == x.sizes() && act_dtype(out),
+              "kgc.residual_group_norm: out [rows, W]");
+  const int64_t rows = x.size(0), W = x.size(1);
+  TORCH_CHECK(groups >= 1 && groups <= 64 && W % groups == 0 && w.numel() == W,
+              "kgc.residual_group_norm: groups / weight");
+  const void* yp = nullptr;
+  if (y.has_value()) {
+    TORCH_CHECK(y->is_contiguous() && y->sizes() == x.sizes() &&
+                y->scalar_type() == out.scalar_type() && y->device() == x.device(),
+                "kgc.residual_group_norm: y");
+    yp = y->data_ptr();
+  }
+  kgc::launch_residual_group_norm(dt_code(out), out.data_ptr(), x.data_ptr<float>(), yp,
+                                  w.data_ptr<float>(), (int)rows, (int)W, (int)groups,
+                                  (float)eps, stream());
+}
+
+void depth_mix_norm(Tensor out, Tensor x, Tensor hist, Tensor y, Tensor coef, Tensor w,
+                    int64_t layer, int64_t groups, double eps) {
+  check_f32(x, "x");
+  check_f32(hist, "hist");
+  check_f32(coef, "coef");
+  check_f32(w, "w");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+  TORCH_CHECK(x.dim() == 2 && hist.dim() == 3, "kgc.depth_mix_norm: x [rows, W], hist [L+1, cap, W]");
+  const int64_t rows = x.size(0), W = x.size(1);
+  TORCH_CHECK(hist.size(2) == W && hist.size(1) >= rows && layer >= 0 && layer + 2 <= hist.size(0) &&
+              coef.numel() >= layer + 2, "kgc.depth_mix_norm: hist / coef extents");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes() && act_dtype(out) &&
+              y.is_contiguous() && y.sizes() == x.sizes() && y.scalar_type() == out.scalar_type() &&
+              y.device() == x.device(), "kgc.depth_mix_norm: out / y");
+  TORCH_CHECK(groups >= 1 && groups <= 64 && W % groups == 0 && w.numel() == W,
+              "kgc.depth_mix_norm: groups / weight");
+  kgc::launch_depth_mix_norm(dt_code(out), out.data_ptr(), x.data_ptr<float>(),
+                             hist.data_ptr<float>(), y.data_ptr(), coef.data_ptr<float>(),
+                             w.data_ptr<float>(), (int)layer, hist.stride(0), (int)rows, (int)W,
+                             (int)groups, (float)eps, stream());
+}
+
+void head_norm_gate(Tensor out, Tensor o, Tensor gt, Tensor w, int64_t H, double eps) {
+  check_f32(o, "o");
+  check_f32(w, "w");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(o.device());
+  TORCH_CHECK(o.dim() == 2 && H >= 1 && H <= 65535 && o.size(1) % H == 0, "kgc.head_norm_gate: o");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == o.sizes() && act_dtype(out), "out");
+  TORCH_CHECK(gt.dim() == 2 && gt.sizes() == o.sizes() && gt.stride(1) == 1 &&
+              gt.scalar_type() == out.scalar_type() && gt.device() == o.device(),
+              "kgc.head_norm_gate: gate slice");
+  TORCH_CHECK(w.numel() == o.size(1), "kgc.head_norm_gate: weight");
+  kgc::launch_head_norm_gate(dt_code(out), out.data_ptr(), o.data_ptr<float>(), gt.data_ptr(),
+                             gt.stride(0), w.data_ptr<float>(), (int)o.size(0), (int)H,
+                             (int)(o.size(1) / H), (float)eps, stream());
+}
+
+void xielu(Tensor out, Tensor z, Tensor ab) {
+  check_gpu(z, "z");
+  check_f32(ab, "ab");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(z.device());
+  TORCH_CHECK(z.is_contiguous() && out.is_contiguous() && out.sizes() == z.sizes() &&
+              out.scalar_type() == z.scalar_type() && act_dtype(z) && ab.numel() == 2,
+              "kgc.xielu: shapes / dtypes");
+  kgc::launch_xielu(dt_code(z), out.data_ptr(), z.data_ptr(), ab.data_ptr<float>(), z.numel(),
+                    stream());
+}
+
+void gate_proj(Tensor out, Tensor h, Tensor w, std::optional<Tensor> bias, int64_t kind_a,
+               int64_t kind_b, int64_t split, double cap) {
+  check_gpu(h, "h");
+  check_f32(out, "out");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
+  TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && w.dim() == 2 && w.is_contiguous() &&
+              w.size(1) == h.size(1) && w.scalar_type() == h.scalar_type() && act_dtype(h) &&
+              w.device() == h.device(), "kgc.gate_proj: h [rows, W], w [N, W]");
+  const int64_t W = h.size(1), N = w.size(0);
+  TORCH_CHECK(W * 4 <= 64 * 1024, "kgc.gate_proj: W <= 16384");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == h.size(0) && out.size(1) == N, "kgc.gate_proj: out");
+  TORCH_CHECK(kind_a >= 0 && kind_a <= 2 && kind_b >= 0 && kind_b <= 2 && cap > 0, "kinds / cap");
+  const float* bp = nullptr;
+  if (bias.has_value()) {
+    check_f32(*bias, "bias");
+    TORCH_CHECK(bias->numel() == N, "kgc.gate_proj: bias");
+    bp = bias->data_ptr<float>();
+  }
+  kgc::launch_gate_proj(dt_code(h), out.data_ptr<float>(), h.data_ptr(), w.data_ptr(), bp,
+                        (int)h.size(0), (int)W, (int)N, (int)kind_a, (int)kind_b, (int)split,
+                        (float)cap, stream());
+}
+
+void check_plain_cache(const Tensor& kc, const Tensor& vc, const Tensor& like, int64_t G,
+                       int64_t dk, int64_t dv) {
+  TORCH_CHECK(kc.dim() == 4 && vc.dim() == 4 && kc.is_contiguous() && vc.is_contiguous() &&
+              kc.size(0) == vc.size(0) && kc.size(1) == G && vc.size(1) == G &&
+              kc.size(2) == vc.size(2) && kc.size(3) == dk && vc.size(3) == dv,
+              "kgc: paged cache k [nb, G, bs, dk], v [nb, G, bs, dv]");
+  TORCH_CHECK(kc.scalar_type() == like.scalar_type() && vc.scalar_type() == like.scalar_type() &&
+              kc.device() == like.device() && vc.device() == like.device(),
+              "kgc: cache dtype / device must match the activations");
+  TORCH_CHECK(kc.size(0) * G * kc.size(2) < (int64_t(1) << 31), "kgc: cache rows exceed int32");
+}
+
+void rope_kv_store(Tensor qkv, Tensor positions, std::optional<Tensor> table, Tensor q_out,
+                   Tensor k_cache, Tensor v_cache, Tensor slots, int64_t H, int64_t G, int64_t dk,
+                   int64_t dv) {
+  check_gpu(qkv, "qkv");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
+  TORCH_CHECK(qkv.dim() == 2 && qkv.stride(1) == 1 && act_dtype(qkv) &&
+              qkv.size(1) >= (H + G) * dk + G * dv, "kgc.rope_kv_store: qkv [T, Hdk + Gdk + Gdv]");
+  const int64_t T = qkv.size(0);
+  check_plain_cache(k_cache, v_cache, qkv, G, dk, dv);
+  TORCH_CHECK(q_out.is_contiguous() && q_out.numel() == T * H * dk &&
+              q_out.scalar_type() == qkv.scalar_type(), "kgc.rope_kv_store: q_out");
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.numel() == T &&
+              positions.is_contiguous() && slots.scalar_type() == at::kLong &&
+              slots.numel() == T && slots.is_contiguous() && positions.is_cuda() && slots.is_cuda(),
+              "kgc.rope_kv_store: positions / slots int64 [T]");
+  const float* tp = nullptr;
+  int64_t rot = 0, rows = 0;
+  if (table.has_value()) {
+    check_f32(*table, "table");
+    TORCH_CHECK(table->dim() == 2 && table->size(1) % 2 == 0 && table->size(1) <= dk,
+                "kgc.rope_kv_store: table [max_pos, rot]");
+    tp = table->data_ptr<float>();
+    rot = table->size(1);
+    rows = table->size(0);
+  }
+  kgc::launch_rope_kv_store(dt_code(qkv), qkv.data_ptr(), qkv.stride(0),
+                            positions.data_ptr<int64_t>(), tp, (int)rot, (int)rows,
+                            q_out.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                            slots.data_ptr<int64_t>(), (int)T, (int)H, (int)G, (int)dk, (int)dv,
+                            (int)k_cache.size(2), (int)k_cache.size(0), stream());
+}
+
+const int* i32_ptr(const std::optional<Tensor>& t, int64_t min_numel, const char* name) {
+  if (!t.has_value()) {
+    TORCH_CHECK(min_numel == 0, "kgc: ", name, " missing");
+    return nullptr;
+  }
+  TORCH_CHECK(t->is_cuda() && t->scalar_type() == at::kInt && t->numel() >= min_numel, "kgc: ",
+              name, " must be int32 on the GPU with >= ", min_numel, " entries");
+  return t->data_ptr<int>();
+}
+
+int64_t table_stride(const std::optional<Tensor>& bt, int64_t rows, int64_t other) {
+  if (!bt.has_value() || rows == 0) return other;
+  TORCH_CHECK(bt->dim() == 2 && bt->size(0) >= rows && bt->stride(1) == 1,
+              "kgc: block tables [rows, max_blocks]");
+  return bt->stride(0);
+}
+
+void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
+                      std::optional<Tensor> qsl, std::optional<Tensor> seq_lens,
+                      std::optional<Tensor> pbt, std::optional<Tensor> ctx_lens,
+                      std::optional<Tensor> dbt, int64_t P, int64_t D, int64_t Tp, double scale,
+                      int64_t window, int64_t keep_first, std::optional<Tensor> gate) {
+  check_gpu(q, "q");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(q.device());
+  TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && act_dtype(q), "kgc.window_attention: q [T, H, dk]");
+  const int64_t T = q.size(0), H = q.size(1), dk = q.size(2);
+  const int64_t G = k_cache.size(1), dv = v_cache.size(3);
+  check_plain_cache(k_cache, v_cache, q, G, dk, dv);
+  TORCH_CHECK(G >= 1 && H % G == 0 && H <= 65535, "kgc.window_attention: heads");
+  TORCH_CHECK(dk <= 4096 && dv <= kgc::window_attention_max_dv(), "kgc.window_attention: head sizes");
+  TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * dv &&
+              out.scalar_type() == q.scalar_type(), "kgc.window_attention: out [T, H * dv]");
+  TORCH_CHECK(P >= 0 && D >= 0 && Tp >= 0 && Tp + D <= T && (P > 0) == (Tp > 0),
+              "kgc.window_attention: step counts");
+  // rows past Tp + D (none in practice) would read ctx_lens out of range: require equality
+  TORCH_CHECK(Tp + D == T, "kgc.window_attention: T must be prefill tokens + decode rows");
+  const int64_t bts = table_stride(pbt, P, table_stride(dbt, D, 0));
+  TORCH_CHECK(table_stride(dbt, D, bts) == bts, "kgc.window_attention: table strides differ");
+  const float* gp = nullptr;
+  if (gate.has_value()) {
+    check_f32(*gate, "gate");
+    TORCH_CHECK(gate->numel() == T * H, "kgc.window_attention: gate [T, H]");
+    gp = gate->data_ptr<float>();
+  }
+  kgc::launch_window_attention(
+      dt_code(q), out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+      i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"), i32_ptr(seq_lens, P, "seq_lens"),
+      i32_ptr(pbt, P, "prefill block tables"), i32_ptr(ctx_lens, D, "ctx_lens"),
+      i32_ptr(dbt, D, "decode block tables"), (int)bts, (int)P, (int)Tp, (int)T, (int)H, (int)G,
+      (int)dk, (int)dv, (int)k_cache.size(2), (int)k_cache.size(0), (float)scale, (int)window,
+      (int)keep_first, gp, stream());
+}
+
+void mlstm_scan(Tensor out, Tensor qkvg, Tensor gates, Tensor S, Tensor n, Tensor m,
+                std::optional<Tensor> qsl, std::optional<Tensor> seq_lens,
+                std::optional<Tensor> ctx_lens, Tensor slots, int64_t P, int64_t D, int64_t Tp,
+                int64_t H, int64_t d, int64_t dv) {
+  check_gpu(qkvg, "qkvg");
+  check_f32(out, "out");
+  check_f32(gates, "gates");
+  check_f32(S, "S");
+  check_f32(n, "n");
+  check_f32(m, "m");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(qkvg.device());
+  TORCH_CHECK(qkvg.dim() == 2 && qkvg.stride(1) == 1 && act_dtype(qkvg) &&
+              qkvg.size(1) >= 2 * H * d + H * dv, "kgc.mlstm_scan: qkvg [T, 2Hd + Hdv ...]");
+  const int64_t T = qkvg.size(0);
+  TORCH_CHECK(Tp + D == T && P >= 0 && D >= 0 && (P > 0) == (Tp > 0), "kgc.mlstm_scan: step counts");
+  TORCH_CHECK(out.numel() == T * H * dv && gates.numel() == T * 2 * H, "kgc.mlstm_scan: out / gates");
+  TORCH_CHECK(d >= 1 && d <= kgc::mlstm_scan_max_dim() && H >= 1 && H <= 65535 && dv >= 1,
+              "kgc.mlstm_scan: head sizes");
+  TORCH_CHECK(S.dim() == 4 && S.size(1) == H && S.size(2) == d && S.size(3) == dv &&
+              n.numel() == S.size(0) * H * d && m.numel() == S.size(0) * H,
+              "kgc.mlstm_scan: state S [slots, H, d, dv], n [slots, H, d], m [slots, H]");
+  kgc::launch_mlstm_scan(dt_code(qkvg), out.data_ptr<float>(), qkvg.data_ptr(), qkvg.stride(0),
+                         gates.data_ptr<float>(), S.data_ptr<float>(), n.data_ptr<float>(),
+                         m.data_ptr<float>(), i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"),
+                         i32_ptr(seq_lens, P, "seq_lens"), i32_ptr(ctx_lens, D, "ctx_lens"),
+                         i32_ptr(slots, P + D, "state slots"), (int)P, (int)D, (int)Tp, (int)H,
+                         (int)d, (int)dv, (int)S.size(0), stream());
+}
+
 }  // namespace
 
 TORCH_LIBRARY(kgc, m) {
+  m.def("residual_group_norm(Tensor(a!) out, Tensor(b!) x, Tensor? y, Tensor w, int groups, float eps) -> ()");
+  m.def("depth_mix_norm(Tensor(a!) out, Tensor(b!) x, Tensor(c!) hist, Tensor y, Tensor coef, Tensor w, "
+        "int layer, int groups, float eps) -> ()");
+  m.def("head_norm_gate(Tensor(a!) out, Tensor o, Tensor g, Tensor w, int H, float eps) -> ()");
+  m.def("xielu(Tensor(a!) out, Tensor z, Tensor ab) -> ()");
+  m.def("gate_proj(Tensor(a!) out, Tensor h, Tensor w, Tensor? bias, int kind_a, int kind_b, int split, "
+        "float cap) -> ()");
+  m.def("rope_kv_store(Tensor qkv, Tensor positions, Tensor? table, Tensor(a!) q_out, Tensor(b!) k_cache, "
+        "Tensor(c!) v_cache, Tensor slots, int H, int G, int dk, int dv) -> ()");
+  m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor? qsl, "
+        "Tensor? seq_lens, Tensor? pbt, Tensor? ctx_lens, Tensor? dbt, int P, int D, int Tp, float scale, "
+        "int window, int keep_first, Tensor? gate) -> ()");
+  m.def("mlstm_scan(Tensor(a!) out, Tensor qkvg, Tensor gates, Tensor(b!) S, Tensor(c!) n, Tensor(d!) m, "
+        "Tensor? qsl, Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int H, int d, "
+        "int dv) -> ()");
   m.def("rms_norm(Tensor(a!) out, Tensor x, Tensor(b!)? residual, Tensor weight, float eps) -> ()");
   m.def("layer_norm(Tensor(a!) out, Tensor x, Tensor weight, Tensor bias, float eps) -> ()");
   m.def("silu_mul(Tensor(a!) out, Tensor x) -> ()");
@@ -1324,6 +1569,14 @@ TORCH_LIBRARY(kgc, m) {
 }
 
 TORCH_LIBRARY_IMPL(kgc, CUDA, m) {
+  m.impl("residual_group_norm", &residual_group_norm);
+  m.impl("depth_mix_norm", &depth_mix_norm);
+  m.impl("head_norm_gate", &head_norm_gate);
+  m.impl("xielu", &xielu);
+  m.impl("gate_proj", &gate_proj);
+  m.impl("rope_kv_store", &rope_kv_store);
+  m.impl("window_attention", &window_attention);
+  m.impl("mlstm_scan", &mlstm_scan);
   m.impl("rms_norm", &rms_norm);
   m.impl("layer_norm", &layer_norm);
   m.impl("silu_mul", &silu_mul);

@@ -68,7 +68,8 @@ def build(force: bool = False, jobs: int = 8, arch: str = "gfx950", verbose: boo
     os.makedirs(BUILD, exist_ok=True)
     hdr_t = _newest_header()
     common = ["-O3", "-fPIC", "-std=c++17", f"--offload-arch={arch}", "-I", CSRC,
-              "-D__HIP_PLATFORM_AMD__=1", "-Wno-unused-result", "-ffp-contract=fast"]
+              "-D__HIP_PLATFORM_AMD__=1", "-Wno-unused-result", "-ffp-contract=fast",
+              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     if debug:
         common.append("-DKGC_DEBUG=1")
     kern = sorted(glob.glob(os.path.join(CSRC, "kernels", "*.hip")))

@@ -1,0 +1,193 @@
+// Row kernels of the hybrid decoders over an fp32 residual stream:
+//   residual_group_norm  x += y (optional); h = grouped RMSNorm(x) * w
+//   depth_mix_norm       the end of a depth-averaged layer: store the layer's result,
+//                        form the weighted sum of all results so far, norm it for the
+//                        next layer -- one pass over the row instead of three kernels
+//   head_norm_gate       per-head RMS norm of a recurrence output, weight, sigmoid gate
+//   xielu                the xIELU activation
+//   gate_proj            a few fp32 gate outputs per row: act(h . w^T + b)
+// All arithmetic is fp32; T is the activation dtype of h / y (bf16, f16 or fp32).
+// One workgroup per row; a row is walked twice (sum of squares, then scale), the second
+// walk re-reading what the same thread wrote in the first.
+#include "common.h"
+#include "launch.h"
+
+namespace kgc {
+
+namespace {
+
+constexpr int NT = 256;
+constexpr int MAX_GROUPS = 64;
+
+// sum of squares per group -> rsqrt(mean + eps), in rs[0..groups)
+template <typename F>
+__device__ __forceinline__ void group_scales(F&& value, int W, int groups, float eps, float* rs,
+                                             float* scratch) {
+  const int gw = W / groups;
+  for (int g = 0; g < groups; ++g) {
+    float ss = 0.f;
+    for (int c = g * gw + threadIdx.x; c < (g + 1) * gw; c += NT) {
+      const float v = value(c);
+      ss += v * v;
+    }
+    ss = block_sum<NT>(ss, scratch);
+    if (threadIdx.x == 0) rs[g] = 1.f / sqrtf(ss / (float)gw + eps);
+  }
+  __syncthreads();
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void residual_group_norm_kernel(
+    T* __restrict__ out, float* __restrict__ x, const T* __restrict__ y,
+    const float* __restrict__ w, int W, int groups, float eps) {
+  __shared__ float rs[MAX_GROUPS];
+  __shared__ float scratch[NT / 64];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * W;
+  if (y != nullptr) {
+    const T* yr = y + row * W;
+    for (int c = threadIdx.x; c < W; c += NT) xr[c] += to_f(yr[c]);
+  }
+  group_scales([&](int c) { return xr[c]; }, W, groups, eps, rs, scratch);
+  const int gw = W / groups;
+  T* o = out + row * W;
+  for (int c = threadIdx.x; c < W; c += NT) o[c] = from_f<T>(xr[c] * rs[c / gw] * w[c]);
+}
+
+// hist [L + 1, Tcap, W]; layer result -> hist[layer + 1]; x = sum_j coef[j] hist[j]
+template <typename T>
+__global__ __launch_bounds__(NT) void depth_mix_norm_kernel(
+    T* __restrict__ out, float* __restrict__ x, float* __restrict__ hist,
+    const T* __restrict__ y, const float* __restrict__ coef, const float* __restrict__ w,
+    int layer, int64_t hist_stride, int W, int groups, float eps) {
+  __shared__ float rs[MAX_GROUPS];
+  __shared__ float scratch[NT / 64];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * W;
+  const T* yr = y + row * W;
+  float* hr = hist + row * W;
+  const float own = coef[layer + 1];
+  for (int c = threadIdx.x; c < W; c += NT) {
+    const float r = xr[c] + to_f(yr[c]);
+    hr[(int64_t)(layer + 1) * hist_stride + c] = r;
+    float acc = 0.f;
+    for (int j = 0; j <= layer; ++j) acc += coef[j] * hr[(int64_t)j * hist_stride + c];
+    xr[c] = acc + own * r;
+  }
+  group_scales([&](int c) { return xr[c]; }, W, groups, eps, rs, scratch);
+  const int gw = W / groups;
+  T* o = out + row * W;
+  for (int c = threadIdx.x; c < W; c += NT) o[c] = from_f<T>(xr[c] * rs[c / gw] * w[c]);
+}
+
+// grid (rows, H), 64 threads: o fp32 [rows, H * dv]; g [rows, g_stride] (column slice)
+template <typename T>
+__global__ __launch_bounds__(64) void head_norm_gate_kernel(
+    T* __restrict__ out, const float* __restrict__ o, const T* __restrict__ g, int64_t g_stride,
+    const float* __restrict__ w, int H, int dv, float eps) {
+  const int64_t row = blockIdx.x;
+  const int h = blockIdx.y;
+  const float* orow = o + (row * H + h) * dv;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < dv; c += 64) ss += orow[c] * orow[c];
+  ss = wave_sum(ss);
+  const float r = 1.f / sqrtf(ss / (float)dv + eps);
+  const T* gr = g + row * g_stride + h * dv;
+  T* orr = out + (row * H + h) * dv;
+  for (int c = threadIdx.x; c < dv; c += 64) {
+    const float gate = 1.f / (1.f + expf(-to_f(gr[c])));
+    orr[c] = from_f<T>(orow[c] * r * w[h * dv + c] * gate);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void xielu_kernel(T* __restrict__ out, const T* __restrict__ z,
+                                                   const float* __restrict__ ab, int64_t n) {
+  const float a = ab[0], b = ab[1];
+  for (int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x; i < n; i += (int64_t)gridDim.x * NT) {
+    const float v = to_f(z[i]);
+    const float r = v > 0.f ? a * v * v + 0.5f * v : b * (expm1f(v) - v) + 0.5f * v;
+    out[i] = from_f<T>(r);
+  }
+}
+
+__device__ __forceinline__ float gate_act(float y, int kind, float cap) {
+  if (kind == 0) return 1.f / (1.f + expf(-y));
+  y = cap * tanhf(y / cap);
+  if (kind == 1) return y;
+  // logsigmoid(y) = min(y, 0) - log1p(exp(-|y|))
+  return fminf(y, 0.f) - log1pf(expf(-fabsf(y)));
+}
+
+// one workgroup per row; the row of h sits in LDS as fp32, each wave takes outputs
+// n = wave, wave + 4, ...
+template <typename T>
+__global__ __launch_bounds__(NT) void gate_proj_kernel(
+    float* __restrict__ out, const T* __restrict__ h, const T* __restrict__ w,
+    const float* __restrict__ bias, int W, int N, int kind_a, int kind_b, int split, float cap) {
+  extern __shared__ float hrow[];
+  const int64_t row = blockIdx.x;
+  const T* hr = h + row * W;
+  for (int c = threadIdx.x; c < W; c += NT) hrow[c] = to_f(hr[c]);
+  __syncthreads();
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int n = wave; n < N; n += NT / 64) {
+    const T* wr = w + (int64_t)n * W;
+    float acc = 0.f;
+    for (int c = lane; c < W; c += 64) acc += hrow[c] * to_f(wr[c]);
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      if (bias != nullptr) acc += bias[n];
+      out[row * N + n] = gate_act(acc, n < split ? kind_a : kind_b, cap);
+    }
+  }
+}
+
+}  // namespace
+
+#define KGC_DISPATCH_T(dtype, ...)                          \
+  do {                                                      \
+    if ((dtype) == DT_BF16) { typedef bf16 T; __VA_ARGS__; } \
+    else if ((dtype) == DT_F16) { typedef f16 T; __VA_ARGS__; } \
+    else { typedef float T; __VA_ARGS__; }                  \
+  } while (0)
+
+void launch_residual_group_norm(int dtype, void* out, float* x, const void* y, const float* w,
+                                int rows, int W, int groups, float eps, hipStream_t s) {
+  if (rows <= 0) return;
+  KGC_DISPATCH_T(dtype, residual_group_norm_kernel<T><<<rows, NT, 0, s>>>(
+      (T*)out, x, (const T*)y, w, W, groups, eps));
+}
+
+void launch_depth_mix_norm(int dtype, void* out, float* x, float* hist, const void* y,
+                           const float* coef, const float* w, int layer, int64_t hist_stride,
+                           int rows, int W, int groups, float eps, hipStream_t s) {
+  if (rows <= 0) return;
+  KGC_DISPATCH_T(dtype, depth_mix_norm_kernel<T><<<rows, NT, 0, s>>>(
+      (T*)out, x, hist, (const T*)y, coef, w, layer, hist_stride, W, groups, eps));
+}
+
+void launch_head_norm_gate(int dtype, void* out, const float* o, const void* g, int64_t g_stride,
+                           const float* w, int rows, int H, int dv, float eps, hipStream_t s) {
+  if (rows <= 0) return;
+  KGC_DISPATCH_T(dtype, head_norm_gate_kernel<T><<<dim3(rows, H), 64, 0, s>>>(
+      (T*)out, o, (const T*)g, g_stride, w, H, dv, eps));
+}
+
+void launch_xielu(int dtype, void* out, const void* z, const float* ab, int64_t n,
+                  hipStream_t s) {
+  if (n <= 0) return;
+  const int grid = (int)std::min<int64_t>((n + NT - 1) / NT, 256 * 32);
+  KGC_DISPATCH_T(dtype, xielu_kernel<T><<<grid, NT, 0, s>>>((T*)out, (const T*)z, ab, n));
+}
+
+void launch_gate_proj(int dtype, float* out, const void* h, const void* w, const float* bias,
+                      int rows, int W, int N, int kind_a, int kind_b, int split, float cap,
+                      hipStream_t s) {
+  if (rows <= 0) return;
+  const size_t lds = (size_t)W * sizeof(float);
+  KGC_DISPATCH_T(dtype, gate_proj_kernel<T><<<rows, NT, lds, s>>>(
+      out, (const T*)h, (const T*)w, bias, W, N, kind_a, kind_b, split, cap));
+}
+
+}  // namespace kgc

@@ -250,4 +250,34 @@ uint32_t ar_read_err(void* sig);
 void ar_raise_peer_flags(void* sig, int rank, int nranks, uint32_t value, hipStream_t s);
 void ar_err_copy_async(void* sig, uint32_t* host_dst, hipStream_t s);
 
+// ---- hybrid decoders (hybrid_norm.hip, attention_window.hip, recurrent.hip) -------------
+// fp32 residual stream x [rows, W]; `dtype` is the activation type of out / y / h / w
+void launch_residual_group_norm(int dtype, void* out, float* x, const void* y, const float* w,
+                                int rows, int W, int groups, float eps, hipStream_t s);
+void launch_depth_mix_norm(int dtype, void* out, float* x, float* hist, const void* y,
+                           const float* coef, const float* w, int layer, int64_t hist_stride,
+                           int rows, int W, int groups, float eps, hipStream_t s);
+void launch_head_norm_gate(int dtype, void* out, const float* o, const void* g, int64_t g_stride,
+                           const float* w, int rows, int H, int dv, float eps, hipStream_t s);
+void launch_xielu(int dtype, void* out, const void* z, const float* ab, int64_t n, hipStream_t s);
+void launch_gate_proj(int dtype, float* out, const void* h, const void* w, const float* bias,
+                      int rows, int W, int N, int kind_a, int kind_b, int split, float cap,
+                      hipStream_t s);
+void launch_rope_kv_store(int dtype, const void* qkv, int64_t qkv_stride,
+                          const int64_t* positions, const float* table, int rot, int table_rows,
+                          void* q_out, void* k_cache, void* v_cache, const int64_t* slots, int T,
+                          int H, int G, int dk, int dv, int bs, int num_blocks, hipStream_t s);
+int window_attention_max_dv();
+void launch_window_attention(int dtype, void* out, const void* q, const void* k_cache,
+                             const void* v_cache, const int* qsl, const int* seq_lens,
+                             const int* pbt, const int* ctx_lens, const int* dbt, int bt_stride,
+                             int P, int Tp, int T, int H, int G, int dk, int dv, int bs,
+                             int num_blocks, float scale, int window, int keep_first,
+                             const float* gate, hipStream_t s);
+int mlstm_scan_max_dim();
+void launch_mlstm_scan(int dtype, float* out, const void* qkvg, int64_t stride,
+                       const float* gates, float* S, float* nst, float* mst, const int* qsl,
+                       const int* seq_lens, const int* ctx_lens, const int* slots, int P, int D,
+                       int Tp, int H, int d, int dv, int num_slots, hipStream_t s);
+
 }  // namespace kgc
