@@ -1,0 +1,346 @@
+"""Dilavik through the engine (registry, safetensors loading, block manager, state slots,
+step packing, kernels) against the plain numpy oracle in ``dilavik_oracle.py``.
+
+Every test writes its own small config.json + model.safetensors (random bf16 weights)
+and drives the engine with the teacher-forced replayer or the generation entry points.
+CPU runs use the reference ops in fp32; ``-m gpu`` runs use the HIP kernels in fp32 and
+bf16.  Windows and pages are small (window 5..9, 8-token pages), so one key wrongly seen
+or missed changes the logits far beyond the tolerances."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import dilavik_oracle as oracle
+from kubernetes_gpu_cluster_amd.engine.config import EngineConfig
+from kubernetes_gpu_cluster_amd.engine.llm_engine import LLM, LLMEngine
+from kubernetes_gpu_cluster_amd.engine.replay import TraceReplayer
+from kubernetes_gpu_cluster_amd.engine.sequence import SamplingParams
+
+CPU = pytest.param("cpu", "float32", id="cpu-fp32")
+GPU32 = pytest.param("cuda", "float32", marks=pytest.mark.gpu, id="gpu-fp32")
+GPU16 = pytest.param("cuda", "bfloat16", marks=pytest.mark.gpu, id="gpu-bf16")
+DEVICES = [CPU, GPU32, GPU16]
+# fp32: every row within 3e-4 of the oracle (relative, mean taken off).  bf16: rounding
+# alone moves a sensitive row by up to ~0.1 with these weights (the CPU reference ops in
+# bf16 show the same), so the rows' median must stay within 0.03 and the worst within 0.3;
+# one key wrongly seen or hidden moves the median beyond 0.3.
+TOL = {"float32": 3e-4, "bfloat16": 0.3}
+TOL_MEDIAN = {"float32": 3e-4, "bfloat16": 0.03}
+
+
+def att(heads=4, kv=2, dim=24, vdim=16, rot=12, base=100.0, size=7, keep=2, scale=0.3, ff=64):
+    return {"type": "attention",
+            "mixer": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": vdim, "scale": scale,
+                      "rot": {"dims": rot, "base": base}, "mask": {"size": size, "keep_first": keep}},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def mls(heads=2, dim=12, vdim=20, cap=8.0, ff=0):
+    return {"type": "mlstm", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "gate_cap": cap},
+            "mlp": {"kind": "dense", "ff": ff} if ff else None}
+
+
+def config(layers, width=96, vocab=160, groups=3, eps=1e-5, scale=6.0):
+    return {"architecture": "Dilavik", "vocab": vocab, "width": width, "layers": layers,
+            "norm": {"eps": eps, "groups": groups}, "embedding": {"scale": scale}}
+
+
+MIXED = config([mls(), att(), att(heads=6, kv=3, dim=16, vdim=24, rot=8, size=5, keep=1, ff=48),
+                mls(heads=3, dim=20, vdim=8, cap=5.0)])
+# sizes a model may make equal or 1: one norm group, kv heads = heads, rotary over the whole
+# head, vdim = dim, nothing kept, attention first and last, a feed-forward on the mLSTM layer
+PLAIN = config([att(heads=2, kv=2, dim=16, vdim=16, rot=16, size=6, keep=0, ff=0),
+                mls(heads=1, dim=16, vdim=16, ff=32), att(heads=3, kv=1, dim=8, vdim=8, rot=2, size=9,
+                                                          keep=3, ff=32)],
+               width=64, vocab=96, groups=1, scale=1.0)
+
+
+def write_model(path, cfg, seed):
+    """Random bf16 weights in the checkpoint's naming; returns them as float64 arrays."""
+    from safetensors.torch import save_file
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    t = {}
+
+    def lin(name, out, inp, gain=1.0):
+        t[name] = torch.randn(out, inp, generator=g) * gain / inp ** 0.5
+
+    def vec(name, n, base, spread):
+        t[name] = base + spread * torch.randn(n, generator=g)
+    t["embed"] = torch.randn(cfg["vocab"], W, generator=g) * 0.5
+    lin("head", cfg["vocab"], W, 2.0)
+    vec("final.norm", W, 1.0, 0.2)
+    for i, lc in enumerate(cfg["layers"]):
+        L, m = "l%d." % i, lc["mixer"]
+        vec(L + "norm1", W, 1.0, 0.2)
+        H, d, dv = m["heads"], m["dim"], m["vdim"]
+        if lc["type"] == "attention":
+            lin(L + "mix.q", H * d, W, 2.0)
+            lin(L + "mix.k", m["kv_heads"] * d, W, 2.0)
+            lin(L + "mix.v", m["kv_heads"] * dv, W)
+            lin(L + "mix.g", H, W, 2.0)
+        else:
+            lin(L + "mix.q", H * d, W, 2.0)
+            lin(L + "mix.k", H * d, W, 2.0)
+            lin(L + "mix.v", H * dv, W)
+            lin(L + "mix.g", H * dv, W)
+            vec(L + "mix.norm", H * dv, 1.0, 0.2)
+            lin(L + "mix.i", H, W, 3.0)
+            lin(L + "mix.f", H, W, 3.0)
+            vec(L + "mix.i.b", H, 0.0, 1.0)
+            vec(L + "mix.f.b", H, 2.0, 1.0)
+        lin(L + "mix.o", W, H * dv)
+        if lc["mlp"]:
+            vec(L + "norm2", W, 1.0, 0.2)
+            lin(L + "mlp.up", lc["mlp"]["ff"], W)
+            lin(L + "mlp.down", W, lc["mlp"]["ff"])
+            t[L + "mlp.act"] = torch.tensor([0.3, -0.4]) + 0.3 * torch.randn(2, generator=g)
+        coef = 0.3 * torch.randn(i + 2, generator=g)
+        coef[-1] += 1.0
+        t[L + "dwa"] = coef
+    t = {k: v.to(torch.bfloat16).contiguous() for k, v in t.items()}
+    os.makedirs(path, exist_ok=True)
+    save_file(t, os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return {k: v.double().numpy() for k, v in t.items()}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = tmp_path_factory.mktemp("dilavik")
+    out = {}
+    for name, cfg, seed in (("mixed", MIXED, 11), ("plain", PLAIN, 12)):
+        d = str(root / name)
+        out[name] = (d, cfg, write_model(d, cfg, seed))
+    return out
+
+
+_engines = {}
+
+
+def engine(models, name, device, dtype, pages=24, page=8, seqs=4, **kw):
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    key = (name, device, dtype, pages, page, seqs, tuple(sorted(kw.items())))
+    if key not in _engines:
+        d = models[name][0]
+        _engines[key] = LLMEngine(EngineConfig(
+            model=d, dtype=dtype, device=device, block_size=page, max_num_seqs=seqs,
+            max_model_len=pages * page, max_num_batched_tokens=pages * page,
+            num_gpu_blocks_override=pages + 1, cuda_graph_max_bs=seqs, **kw))
+    return _engines[key]
+
+
+def row_errs(got, want):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    w = want - want.mean(-1, keepdims=True)
+    return np.sqrt((d ** 2).mean(-1) / (w ** 2).mean(-1))
+
+
+def rel_err(got, want):
+    return float(row_errs(got, want).max())
+
+
+def close(got, want, dtype):
+    e = row_errs(got, want)
+    if len(e) < 8:
+        return bool(e.max() < TOL[dtype])
+    return bool(e.max() < TOL[dtype] and np.median(e) < TOL_MEDIAN[dtype])
+
+
+def tokens_for(cfg, n, seed):
+    return np.random.default_rng(seed).integers(0, cfg["vocab"], n).tolist()
+
+
+def run_alone(rp, rid, toks, cuts):
+    """Feed `toks` in portions of the sizes `cuts` (the last size repeats); all logits."""
+    out, lo, i = [], 0, 0
+    while lo < len(toks):
+        n = cuts[min(i, len(cuts) - 1)]
+        i += 1
+        hi = min(len(toks), lo + n)
+        lg = rp.step([{"id": rid, "tokens": toks[lo:hi], "want": list(range(hi - lo))}],
+                     [rid] if hi == len(toks) else [])
+        out.append(lg.cpu().numpy())
+        lo = hi
+    return np.concatenate(out)
+
+
+# ---------------------------------------------------------------- whole prompts, decode, portions
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "plain"])
+def test_whole_prompt_matches_oracle(models, name, device, dtype):
+    _, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 61, 1)
+    want = oracle.forward(toks, cfg, wts)
+    got = run_alone(rp, "w", toks, [len(toks)])
+    assert close(got, want, dtype)
+    # the first tokens of a sequence, and a one-token prompt
+    assert close(got[:3], want[:3], dtype)
+    one = run_alone(rp, "o", toks[:1], [1])
+    assert close(one, want[:1], dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "plain"])
+def test_prefill_then_token_by_token(models, name, device, dtype):
+    _, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 70, 2)
+    want = oracle.forward(toks, cfg, wts)
+    got = run_alone(rp, "d", toks, [20, 1])        # 50 decoded tokens: every window passes
+    assert close(got, want, dtype)
+    got = run_alone(rp, "e", toks, [1])            # decoding from the very first token
+    assert close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("cuts", [[2], [3, 2, 7, 2, 11, 5, 1], [8], [9, 16, 2, 1]])
+def test_portions(models, device, dtype, cuts):
+    _, cfg, wts = models["mixed"]
+    eng = engine(models, "mixed", device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 45, 3)
+    want = oracle.forward(toks, cfg, wts)
+    assert close(run_alone(rp, "p", toks, cuts), want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_long_decode(models, device, dtype):
+    _, cfg, wts = models["plain"]
+    eng = engine(models, "plain", device, dtype, pages=40)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 150, 4)
+    want = oracle.forward(toks, cfg, wts)
+    got = run_alone(rp, "l", toks, [5, 1])
+    assert close(got[-20:], want[-20:], dtype)
+    assert close(got, want, dtype)
+
+
+# ---------------------------------------------------------------- batches, pages and slots reused
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_mixed_batches_and_reuse(models, device, dtype):
+    """Four live requests of unequal length, portions beside decode rows, requests that
+    sit out steps; the pool (14 pages) and the four slots are used again by later
+    requests.  Every row must match the request run alone (the oracle)."""
+    _, cfg, wts = models["mixed"]
+    eng = engine(models, "mixed", device, dtype, pages=14)
+    rp = TraceReplayer(eng)
+    lens = {"a": 30, "b": 9, "c": 41, "d": 2, "e": 25, "f": 17, "g": 33}
+    toks = {k: tokens_for(cfg, n, 10 + i) for i, (k, n) in enumerate(lens.items())}
+    want = {k: oracle.forward(v, cfg, wts) for k, v in toks.items()}
+    at = {k: 0 for k in lens}
+    got = {k: [] for k in lens}
+    # (request, tokens) per step; a request is freed when its tokens are used up
+    plan = [[("a", 7), ("b", 3)], [("a", 1), ("b", 1), ("c", 12)], [("a", 1), ("c", 2), ("d", 2)],
+            [("b", 5), ("c", 1), ("a", 9)], [("a", 1), ("c", 1)], [("a", 11), ("c", 25), ("e", 4)],
+            [("e", 1), ("f", 17)], [("e", 1), ("g", 8)], [("e", 19), ("g", 1)], [("g", 24)]]
+    used_slots, used_pages = set(), []
+    for step in plan:
+        entries, end = [], []
+        for k, n in step:
+            lo = at[k]
+            entries.append({"id": k, "tokens": toks[k][lo:lo + n], "want": list(range(n))})
+            at[k] += n
+            if at[k] == lens[k]:
+                end.append(k)
+        live = dict(rp.seqs)
+        lg = rp.step(entries, end).cpu().numpy()
+        for k, s in rp.seqs.items():
+            used_slots.add(s.slot)
+            used_pages += s.block_ids
+        o = 0
+        for k, n in step:
+            got[k].append(lg[o:o + n])
+            o += n
+        assert len(live) <= 4
+    assert all(at[k] == lens[k] for k in lens)
+    assert len(used_pages) > len(set(used_pages)) and len(set(used_pages)) <= 14
+    for k in lens:
+        assert close(np.concatenate(got[k]), want[k], dtype), k
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_slot_reuse_starts_from_zero_state(models, device, dtype):
+    """A slot that held a long request is given to a new one: its recurrent state and its
+    pages must not leak into the new request's first tokens."""
+    _, cfg, wts = models["mixed"]
+    eng = engine(models, "mixed", device, dtype, seqs=1, pages=10)
+    rp = TraceReplayer(eng)
+    first, second = tokens_for(cfg, 50, 20), tokens_for(cfg, 12, 21)
+    run_alone(rp, "x", first, [50])
+    got = run_alone(rp, "y", second, [4, 1])
+    assert close(got, oracle.forward(second, cfg, wts), dtype)
+
+
+# ---------------------------------------------------------------- residual stream per layer
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_layer_taps(models, device, dtype):
+    d, cfg, wts = models["mixed"]
+    eng = engine(models, "mixed", device, dtype)
+    runner = eng.executor.runner
+    toks = tokens_for(cfg, 19, 5)
+    want = []
+    oracle.forward(toks, cfg, wts, want)
+    rp = TraceReplayer(eng)
+    taps = []
+    model = runner.model
+    orig = model.forward
+    model.forward = lambda *a, **k: orig(*a, taps=taps, **k)
+    try:
+        run_alone(rp, "t", toks, [len(toks)])
+    finally:
+        model.forward = orig
+    assert len(taps) == len(want)
+    tol = 2e-4 if dtype == "float32" else 0.05
+    for got, w in zip(taps, want):
+        g = got.cpu().double().numpy()
+        assert np.abs(g - w).max() <= tol * np.abs(w).max()
+
+
+# ---------------------------------------------------------------- generation entry points
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_greedy_generation_through_scheduler(models, device, dtype):
+    """LLM.generate (request intake, continuous batching, chunked prefill with a token
+    budget smaller than the prompts, sampling at temperature 0): every generated token is
+    the oracle's argmax given the tokens before it."""
+    d, cfg, wts = models["mixed"]
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    llm = LLM(model=d, dtype=dtype, device=device, block_size=8, max_num_seqs=3,
+              max_model_len=96, max_num_batched_tokens=16, num_gpu_blocks_override=40,
+              cuda_graph_max_bs=3)
+    try:
+        prompts = [tokens_for(cfg, n, 30 + n) for n in (5, 23, 1, 37, 12)]
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    finally:
+        llm.shutdown()
+    margin = 1e-3 if dtype == "float32" else 0.15
+    for p, o in zip(prompts, outs):
+        gen = list(o.output_token_ids)
+        assert len(gen) == 12
+        lg = oracle.forward(p + gen, cfg, wts)
+        for i, tok in enumerate(gen):
+            row = lg[len(p) - 1 + i]
+            assert row[tok] >= row.max() - margin * (row.max() - row.min()), (i, tok)
+
+
+def test_registry_and_config_reader(models):
+    from kubernetes_gpu_cluster_amd.models import resolve_model
+    d, cfg, _ = models["mixed"]
+    mc, wdir = resolve_model(d)
+    assert mc.arch == "dilavik" and wdir == d and mc.num_layers == 4
+    assert [s.kind for s in mc.layer_specs] == ["mlstm", "attention", "attention", "mlstm"]
+    sp = mc.layer_specs[2]
+    assert (sp.heads, sp.kv_heads, sp.dim, sp.vdim, sp.rot_dims, sp.ff) == (6, 3, 16, 24, 8, 48)
+    assert (sp.window.size, sp.window.keep_first) == (5, 1)
+    assert mc.has_recurrent_state and mc.norm_groups == 3 and mc.embed_scale == 6.0
