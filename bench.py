@@ -88,7 +88,11 @@ def parse():
     ap.add_argument("--no-prefill-first", dest="prefill_first", action="store_false")
     ap.add_argument("--log-level", default="WARNING",
                     help="python logging level on stderr (INFO shows the GEMM tuner's choices)")
-    ap.add_argument("--mode", default="service", choices=["service", "engine"],
+    ap.add_argument("--compare-sizes", default="w2048,w4096",
+                    help="--mode compare: size suffixes of the dilavik-* / llama-* preset pairs")
+    ap.add_argument("--compare-families", default="dilavik,llama",
+                    help="--mode compare: which preset of each pair to run (profiling one alone)")
+    ap.add_argument("--mode", default="service", choices=["service", "engine", "compare"],
                     help="service: HTTP/SSE through API server + router (headline); "
                          "engine: LLMEngine.step() in-process")
     ap.add_argument("--api-server-count", type=int, default=0,
@@ -588,6 +592,78 @@ def _comm_probe(rank: int, world: int, local_rank: int, timeout_s: float = 240.0
             os.remove(out)
 
 
+def _compare_one(model: str, args) -> dict:
+    """Prefill and decode throughput of one preset through LLMEngine.step(): a prefill-only
+    wave (every request stops after its first token), then a wave whose decode phase is
+    timed from the moment every request has its first token."""
+    from kubernetes_gpu_cluster_amd.engine.config import EngineConfig
+    from kubernetes_gpu_cluster_amd.engine.llm_engine import LLMEngine
+    from kubernetes_gpu_cluster_amd.engine.sequence import SamplingParams
+    eng = LLMEngine(EngineConfig(
+        model=model, dtype=args.dtype, max_model_len=args.max_model_len,
+        max_num_seqs=args.max_num_seqs, max_num_batched_tokens=args.max_num_batched_tokens,
+        gpu_memory_utilization=args.gpu_memory_utilization, enforce_eager=args.enforce_eager,
+        random_init=True, seed=0, enable_prefix_caching=False))
+    vocab = eng.mcfg.vocab_size
+    g = torch.Generator().manual_seed(7)
+
+    def wave(n, in_len, out_len):
+        sp = SamplingParams(temperature=args.temperature, max_tokens=out_len, ignore_eos=True)
+        t0 = time.monotonic()
+        seqs = [eng.add_request(torch.randint(10, vocab - 10, (in_len,), generator=g).tolist(), sp,
+                                arrival_time=t0) for _ in range(n)]
+        while eng.has_unfinished():
+            eng.step()
+        torch.cuda.synchronize()
+        t1 = time.monotonic()
+        first = max(s.first_token_time for s in seqs)
+        out = sum(len(s.output_token_ids) for s in seqs)
+        return t1 - t0, first, t1, out
+
+    n, L, K = args.num_prompts, args.input_len, args.output_len
+    res = {"model": model, "params_M": round(eng.mcfg.num_params() / 1e6, 1)}
+    for _ in range(max(1, args.warmup)):
+        wave(min(n, 32), L, 4)
+    pre, dec = [], []
+    for _ in range(max(1, args.steps)):
+        dt, _, _, _ = wave(n, L, 1)
+        pre.append(n * L / dt)
+        _, first, t1, out = wave(n, L, K)
+        dec.append((out - n) / (t1 - first))
+    res["prefill_tok_s"] = round(statistics.median(pre), 1)
+    res["decode_tok_s"] = round(statistics.median(dec), 1)
+    res["graph_steps"] = eng.executor.runner.stats["graph_steps"]
+    eng.shutdown()
+    del eng
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    return res
+
+
+def main_compare(args):
+    """--mode compare: the hybrid presets beside the Llama-style decoders of equal size
+    (models/configs.py), same requests, same engine settings, one JSON line per model and a
+    closing line with the ratios.  Random weights, synthetic prompts."""
+    assert torch.cuda.is_available(), "bench.py --mode compare needs a GPU"
+    rows = []
+    for size in args.compare_sizes.split(","):
+        pair = {}
+        for fam in args.compare_families.split(","):
+            r = _compare_one(f"{fam}-{size}", args)
+            r.update(batch=args.num_prompts, input_len=args.input_len, output_len=args.output_len,
+                     dtype=args.dtype)
+            print(json.dumps(r), flush=True)
+            pair[fam] = r
+        if len(pair) == 2:
+            rows.append({"size": size,
+                         "prefill_ratio": round(pair["dilavik"]["prefill_tok_s"] /
+                                                pair["llama"]["prefill_tok_s"], 3),
+                         "decode_ratio": round(pair["dilavik"]["decode_tok_s"] /
+                                               pair["llama"]["decode_tok_s"], 3)})
+    print(json.dumps({"mode": "compare", "data": "synthetic", "weights": "random", "ratios": rows}))
+
+
 def failed_any(parts) -> bool:
     return any(p["failed"] for p in parts)
 
@@ -596,6 +672,8 @@ def main():
     args = parse()
     if args.mode == "engine":
         main_engine(args)
+    elif args.mode == "compare":
+        main_compare(args)
     else:
         main_service(args)
 

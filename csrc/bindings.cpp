@@ -1381,8 +1381,10 @@ int64_t table_stride(const std::optional<Tensor>& bt, int64_t rows, int64_t othe
 void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
                       std::optional<Tensor> qsl, std::optional<Tensor> seq_lens,
                       std::optional<Tensor> pbt, std::optional<Tensor> ctx_lens,
-                      std::optional<Tensor> dbt, int64_t P, int64_t D, int64_t Tp, double scale,
-                      int64_t window, int64_t keep_first, std::optional<Tensor> gate) {
+                      std::optional<Tensor> dbt, std::optional<Tensor> work_seq,
+                      std::optional<Tensor> work_blk, int64_t P, int64_t D, int64_t Tp,
+                      double scale, int64_t window, int64_t keep_first,
+                      std::optional<Tensor> gate, bool fast) {
   check_gpu(q, "q");
   c10::hip::HIPGuardMasqueradingAsCUDA g(q.device());
   TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && act_dtype(q), "kgc.window_attention: q [T, H, dk]");
@@ -1393,10 +1395,8 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   TORCH_CHECK(dk <= 4096 && dv <= kgc::window_attention_max_dv(), "kgc.window_attention: head sizes");
   TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * dv &&
               out.scalar_type() == q.scalar_type(), "kgc.window_attention: out [T, H * dv]");
-  TORCH_CHECK(P >= 0 && D >= 0 && Tp >= 0 && Tp + D <= T && (P > 0) == (Tp > 0),
-              "kgc.window_attention: step counts");
-  // rows past Tp + D (none in practice) would read ctx_lens out of range: require equality
-  TORCH_CHECK(Tp + D == T, "kgc.window_attention: T must be prefill tokens + decode rows");
+  TORCH_CHECK(P >= 0 && D >= 0 && Tp >= 0 && (P > 0) == (Tp > 0) && Tp + D == T,
+              "kgc.window_attention: T must be prefill tokens + decode rows");
   const int64_t bts = table_stride(pbt, P, table_stride(dbt, D, 0));
   TORCH_CHECK(table_stride(dbt, D, bts) == bts, "kgc.window_attention: table strides differ");
   const float* gp = nullptr;
@@ -1405,13 +1405,40 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
     TORCH_CHECK(gate->numel() == T * H, "kgc.window_attention: gate [T, H]");
     gp = gate->data_ptr<float>();
   }
-  kgc::launch_window_attention(
-      dt_code(q), out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
-      i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"), i32_ptr(seq_lens, P, "seq_lens"),
-      i32_ptr(pbt, P, "prefill block tables"), i32_ptr(ctx_lens, D, "ctx_lens"),
-      i32_ptr(dbt, D, "decode block tables"), (int)bts, (int)P, (int)Tp, (int)T, (int)H, (int)G,
-      (int)dk, (int)dv, (int)k_cache.size(2), (int)k_cache.size(0), (float)scale, (int)window,
-      (int)keep_first, gp, stream());
+  const int* qp = i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc");
+  const int* sp = i32_ptr(seq_lens, P, "seq_lens");
+  const int* pp = i32_ptr(pbt, P, "prefill block tables");
+  const int* cp = i32_ptr(ctx_lens, D, "ctx_lens");
+  const int* dp = i32_ptr(dbt, D, "decode block tables");
+  const int bs = (int)k_cache.size(2), nb = (int)k_cache.size(0), dt = dt_code(q);
+  int rest = 3;                   // row kinds the one-wave kernel still has to run
+  if (fast && P > 0 && work_seq.has_value() && work_blk.has_value() &&
+      kgc::window_prefill_mfma_ok(dt, (int)dk, (int)dv)) {
+    const int64_t nw = work_seq->numel();
+    TORCH_CHECK(work_blk->numel() == nw && work_seq->scalar_type() == at::kInt &&
+                work_blk->scalar_type() == at::kInt && work_seq->is_cuda() && work_blk->is_cuda(),
+                "kgc.window_attention: work list int32 [n] on the GPU");
+    kgc::launch_window_prefill_mfma(dt, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
+                                    v_cache.data_ptr(), qp, sp, pp, (int)bts,
+                                    work_seq->data_ptr<int>(), work_blk->data_ptr<int>(), (int)nw,
+                                    kgc::prefill_block_m(), (int)H, (int)G, (int)dk, (int)dv, bs,
+                                    nb, (float)scale, (int)window, (int)keep_first, gp, stream());
+    rest &= ~1;
+  }
+  if (fast && D > 0 && kgc::window_decode_ok((int)dk, (int)dv, (int)(H / G)) &&
+      kgc::window_decode_lds((int)dk, (int)dv, (int)(H / G)) <= 64 * 1024) {
+    kgc::launch_window_decode(dt, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
+                              v_cache.data_ptr(), cp, dp, (int)bts, (int)Tp, (int)D, (int)H,
+                              (int)G, (int)dk, (int)dv, bs, nb, (float)scale, (int)window,
+                              (int)keep_first, gp, stream());
+    rest &= ~2;
+  }
+  if (!P) rest &= ~1;
+  if (!D) rest &= ~2;
+  kgc::launch_window_attention(dt, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
+                               v_cache.data_ptr(), qp, sp, pp, cp, dp, (int)bts, (int)P, (int)Tp,
+                               (int)T, (int)H, (int)G, (int)dk, (int)dv, bs, nb, (float)scale,
+                               (int)window, (int)keep_first, gp, rest, stream());
 }
 
 void mlstm_scan(Tensor out, Tensor qkvg, Tensor gates, Tensor S, Tensor n, Tensor m,
@@ -1456,8 +1483,8 @@ TORCH_LIBRARY(kgc, m) {
   m.def("rope_kv_store(Tensor qkv, Tensor positions, Tensor? table, Tensor(a!) q_out, Tensor(b!) k_cache, "
         "Tensor(c!) v_cache, Tensor slots, int H, int G, int dk, int dv) -> ()");
   m.def("window_attention(Tensor(a!) out, Tensor q, Tensor k_cache, Tensor v_cache, Tensor? qsl, "
-        "Tensor? seq_lens, Tensor? pbt, Tensor? ctx_lens, Tensor? dbt, int P, int D, int Tp, float scale, "
-        "int window, int keep_first, Tensor? gate) -> ()");
+        "Tensor? seq_lens, Tensor? pbt, Tensor? ctx_lens, Tensor? dbt, Tensor? work_seq, Tensor? work_blk, "
+        "int P, int D, int Tp, float scale, int window, int keep_first, Tensor? gate, bool fast) -> ()");
   m.def("mlstm_scan(Tensor(a!) out, Tensor qkvg, Tensor gates, Tensor(b!) S, Tensor(c!) n, Tensor(d!) m, "
         "Tensor? qsl, Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int H, int d, "
         "int dv) -> ()");

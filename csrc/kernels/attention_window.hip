@@ -71,8 +71,9 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
     const T* __restrict__ v_cache, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const int* __restrict__ pbt, const int* __restrict__ ctx_lens, const int* __restrict__ dbt,
     int bt_stride, int P, int Tp, int H, int G, int dk, int dv, int bs, int num_blocks,
-    float scale, int window, int keep_first, const float* __restrict__ gate) {
+    float scale, int window, int keep_first, const float* __restrict__ gate, int kinds) {
   extern __shared__ float lds[];
+  if (!(kinds & (blockIdx.x < Tp ? 1 : 2))) return;   // rows another kernel of the step owns
   float* qs = lds;                  // [dk]
   float* pw = lds + dk;             // [64]
   int* voff = (int*)(pw + 64);      // [64] (block * G + g) * bs + row
@@ -152,6 +153,389 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
   }
 }
 
+// ---- 8 consecutive elements of a cache row as fp32 (16-byte loads; dk % 8 == 0)
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
+  if constexpr (std::is_same_v<T, float>) {
+    const float4 a = *reinterpret_cast<const float4*>(p);
+    const float4 b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  } else {
+    Pack8<T> t;
+    t.u = *reinterpret_cast<const u32x4*>(p);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = to_f(t.h[e]);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void load2(const T* p, float& a, float& b) {
+  if constexpr (std::is_same_v<T, float>) {
+    const float2 t = *reinterpret_cast<const float2*>(p);
+    a = t.x;
+    b = t.y;
+  } else {
+    union { uint32_t u; T h[2]; } t;
+    t.u = *reinterpret_cast<const uint32_t*>(p);
+    a = to_f(t.h[0]);
+    b = to_f(t.h[1]);
+  }
+}
+
+// Decode rows: one workgroup of 8 waves per (row, kv head, group of up to QH query heads).
+// The visible keys (kept first tokens + window) are cut into 64-key chunks dealt round-robin
+// to the waves.  In a chunk each lane takes one key: its row is read once (16-byte loads)
+// and dotted with every query head of the group (q in LDS as fp32); then each lane takes
+// two value columns and walks the chunk's 64 value rows, again once for all heads.  Every
+// wave carries its own online-softmax state per head; the eight states merge in LDS in
+// wave order (deterministic).  Scores, weights and sums are fp32.
+constexpr int DEC_WAVES = 8;
+constexpr int DEC_UMAX = 4;          // value columns per lane: 2 * DEC_UMAX * 64 >= dv
+
+template <typename T, int QH>
+__global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
+    T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
+    const T* __restrict__ v_cache, const int* __restrict__ ctx_lens, const int* __restrict__ dbt,
+    int bt_stride, int Tp, int H, int G, int dk, int dv, int bs, int num_blocks, float scale,
+    int window, int keep_first, const float* __restrict__ gate) {
+  extern __shared__ float lds[];
+  const int dd = blockIdx.x, g = blockIdx.y, qpg = H / G, hq0 = blockIdx.z * QH;
+  const int nh = min(QH, qpg - hq0);
+  const int t = Tp + dd, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* qs = lds;                                    // [QH][dk]
+  float* pb = qs + QH * dk;                           // [waves][QH][64]
+  int* ob = (int*)(pb + DEC_WAVES * QH * 64);         // [waves][64]
+  float* mm = (float*)(ob + DEC_WAVES * 64);          // [waves][QH]
+  float* ml = mm + DEC_WAVES * QH;                    // [waves][QH]
+  float* accs = ml + DEC_WAVES * QH;                  // [QH][dv]
+  const int h0 = g * qpg + hq0;                       // first query head of this workgroup
+  const int pos = ctx_lens[dd] - 1;
+  const int* bt = dbt + (int64_t)dd * bt_stride;
+  if (pos < 0 || pos >= bt_stride * bs) {             // a padding row: zeros
+    for (int e = threadIdx.x; e < nh * dv; e += 64 * DEC_WAVES)
+      out[((int64_t)t * H + h0) * dv + e] = from_f<T>(0.f);
+    return;
+  }
+  for (int e = threadIdx.x; e < nh * dk; e += 64 * DEC_WAVES)
+    qs[e] = to_f(q[((int64_t)t * H + h0) * dk + e]);
+  for (int e = threadIdx.x; e < QH * dv; e += 64 * DEC_WAVES) accs[e] = 0.f;
+  __syncthreads();
+  const int lo_w = window > 0 ? max(0, pos - window + 1) : 0;
+  const int ns = min(keep_first, lo_w);
+  const int total = ns + (pos - lo_w + 1);
+  const int nchunks = (total + 63) >> 6;
+  float m[QH], l[QH], acc[QH][DEC_UMAX][2];
+#pragma unroll
+  for (int h = 0; h < QH; ++h) {
+    m[h] = -INFINITY;
+    l[h] = 0.f;
+#pragma unroll
+    for (int u = 0; u < DEC_UMAX; ++u) acc[h][u][0] = acc[h][u][1] = 0.f;
+  }
+  float* pw = pb + wave * QH * 64;
+  int* ow = ob + wave * 64;
+  for (int chunk = wave; chunk < nchunks; chunk += DEC_WAVES) {
+    const int idx = chunk * 64 + lane;
+    const bool ok = idx < total;
+    float sc[QH];
+#pragma unroll
+    for (int h = 0; h < QH; ++h) sc[h] = 0.f;
+    int ro = 0;
+    if (ok) {
+      const int j = idx < ns ? idx : lo_w + (idx - ns);
+      int b = bt[j / bs];
+      if (b < 0 || b >= num_blocks) b = 0;
+      ro = (b * G + g) * bs + (j % bs);
+      const T* kr = k_cache + (int64_t)ro * dk;
+      for (int c = 0; c < dk; c += 8) {
+        float kv[8];
+        load8(kr + c, kv);
+#pragma unroll
+        for (int h = 0; h < QH; ++h) {
+          if (h < nh) {
+            const float* qh = qs + h * dk + c;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sc[h] += qh[e] * kv[e];
+          }
+        }
+      }
+    }
+    float alpha[QH];
+#pragma unroll
+    for (int h = 0; h < QH; ++h) {
+      const float sv = ok ? sc[h] * scale : -INFINITY;
+      const float mn = fmaxf(m[h], wave_max(sv));
+      alpha[h] = expf(m[h] - mn);
+      const float p = ok ? expf(sv - mn) : 0.f;
+      l[h] = l[h] * alpha[h] + wave_sum(p);
+      m[h] = mn;
+      pw[h * 64 + lane] = p;
+    }
+    ow[lane] = ro;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const int cnt = min(64, total - chunk * 64);
+#pragma unroll
+    for (int u = 0; u < DEC_UMAX; ++u) {
+      const int c0 = 2 * lane + 128 * u;
+      if (c0 < dv) {
+        float a0[QH], a1[QH];
+#pragma unroll
+        for (int h = 0; h < QH; ++h) {
+          a0[h] = acc[h][u][0] * alpha[h];
+          a1[h] = acc[h][u][1] * alpha[h];
+        }
+        for (int jj = 0; jj < cnt; ++jj) {
+          float v0, v1;
+          load2(v_cache + (int64_t)ow[jj] * dv + c0, v0, v1);
+#pragma unroll
+          for (int h = 0; h < QH; ++h) {
+            const float p = pw[h * 64 + jj];
+            a0[h] += p * v0;
+            a1[h] += p * v1;
+          }
+        }
+#pragma unroll
+        for (int h = 0; h < QH; ++h) {
+          acc[h][u][0] = a0[h];
+          acc[h][u][1] = a1[h];
+        }
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane == 0) {
+#pragma unroll
+    for (int h = 0; h < QH; ++h) {
+      mm[wave * QH + h] = m[h];
+      ml[wave * QH + h] = l[h];
+    }
+  }
+  __syncthreads();
+  float f[QH];
+#pragma unroll
+  for (int h = 0; h < QH; ++h) {
+    float M = -INFINITY;
+    for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, mm[w * QH + h]);
+    f[h] = m[h] == -INFINITY ? 0.f : expf(m[h] - M);
+  }
+  for (int w = 0; w < DEC_WAVES; ++w) {
+    if (wave == w && nchunks > w) {
+#pragma unroll
+      for (int u = 0; u < DEC_UMAX; ++u) {
+        const int c0 = 2 * lane + 128 * u;
+        if (c0 < dv) {
+#pragma unroll
+          for (int h = 0; h < QH; ++h) {
+            accs[h * dv + c0] += acc[h][u][0] * f[h];
+            accs[h * dv + c0 + 1] += acc[h][u][1] * f[h];
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  for (int e = threadIdx.x; e < nh * dv; e += 64 * DEC_WAVES) {
+    const int h = e / dv;
+    float M = -INFINITY, L = 0.f;
+    for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, mm[w * QH + h]);
+    for (int w = 0; w < DEC_WAVES; ++w) {
+      const float mw = mm[w * QH + h];
+      if (mw != -INFINITY) L += ml[w * QH + h] * expf(mw - M);
+    }
+    const float gt = gate != nullptr ? gate[(int64_t)t * H + h0 + h] : 1.f;
+    out[((int64_t)t * H + h0) * dv + e] = from_f<T>(accs[e] * gt / L);
+  }
+}
+
+// Prefill chunks on the matrix cores (16-bit activations).  One workgroup of 4 waves per
+// (64 query rows of a chunk, query head); wave w owns rows 16 w .. 16 w + 15.  Keys come in
+// 64-key tiles -- first the kept first tokens that lie before the tile's earliest window,
+// then the span from that window's start to the last row -- gathered from the pages into
+// LDS as K [64][dk + 8] and V^T [dv][64 + 8].  Per tile and wave:
+//   S^T = K . Q^T   (v_mfma_f32_16x16x32; the query is lane & 15 in every accumulator, so
+//                    the softmax statistics are lane-local up to two shuffles),
+//   visibility mask, online softmax in fp32,
+//   O^T += V^T . P^T with P^T taken straight from the S^T accumulators (key m of an A row
+//                    is 8 (m >> 2) + (m & 3), + 4 for the second tile of a 32-key pair).
+// The fp32 weights enter that product as a bf16/f16 pair (value + remainder), two MFMAs,
+// so they carry ~16 mantissa bits rather than 8.
+constexpr int PFW_BM = 64, PFW_BN = 64, PFW_KPAD = 8, PFW_VPAD = 8;
+
+template <typename T, int KSM, int DTM>
+__global__ __launch_bounds__(256) void window_prefill_mfma_kernel(
+    T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
+    const T* __restrict__ v_cache, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
+    const int* __restrict__ pbt, int bt_stride, const int* __restrict__ work_seq,
+    const int* __restrict__ work_blk, int blk_rows, int H, int G, int dk, int dv, int bs,
+    int num_blocks, float scale, int window, int keep_first, const float* __restrict__ gate) {
+  typedef typename Vec8<T>::type V8;
+  extern __shared__ float lds_f[];
+  T* Ks = reinterpret_cast<T*>(lds_f);                 // [64][dk + 8]
+  const int kst = dk + PFW_KPAD, vst = PFW_BN + PFW_VPAD;
+  T* Vt = Ks + PFW_BN * kst;                           // [dv][64 + 8]
+  const int item = blockIdx.x / (blk_rows / PFW_BM), sub = blockIdx.x % (blk_rows / PFW_BM);
+  const int seq = work_seq[item], h = blockIdx.y, g = h / (H / G);
+  const int q0 = qsl[seq], qlen = qsl[seq + 1] - q0, ctx0 = seq_lens[seq] - qlen;
+  const int r0 = work_blk[item] * blk_rows + sub * PFW_BM;
+  if (r0 >= qlen || ctx0 < 0) return;
+  const int rows = min(PFW_BM, qlen - r0);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, qd = lane >> 4;
+  const int nks = dk >> 5, ndt = dv >> 4;
+  const int* bt = pbt + (int64_t)seq * bt_stride;
+  const int myrow = r0 + 16 * wave + r16;
+  const bool rowok = myrow < qlen;
+  const int qpos = ctx0 + myrow;
+  // this wave's q fragments: lane (r16, qd) holds dims 32 s + 8 qd .. + 7 of its row
+  V8 qf[KSM];
+  {
+    const T* qrow = q + ((int64_t)(q0 + (rowok ? myrow : r0)) * H + h) * dk;
+#pragma unroll
+    for (int s2 = 0; s2 < KSM; ++s2) {
+      Pack8<T> tq;
+      tq.u = u32x4{0u, 0u, 0u, 0u};
+      if (s2 < nks && rowok) tq.u = *reinterpret_cast<const u32x4*>(qrow + 32 * s2 + 8 * qd);
+      qf[s2] = tq.v;
+    }
+  }
+  f32x4 o[DTM];
+#pragma unroll
+  for (int t2 = 0; t2 < DTM; ++t2) o[t2] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int p_min = ctx0 + r0, p_max = ctx0 + r0 + rows - 1;
+  const int lo_min = window > 0 ? max(0, p_min - window + 1) : 0;
+  const int ns = window > 0 ? min(keep_first, lo_min) : 0;
+  const int nsink = (ns + PFW_BN - 1) / PFW_BN;
+  const int nmain = (p_max - lo_min + PFW_BN) / PFW_BN;
+  // the wave's own span of visible keys (tiles outside it are staged but not computed)
+  const int wp_lo = ctx0 + r0 + 16 * wave, wp_hi = min(wp_lo + 15, p_max);
+  const int w_lo = window > 0 ? max(0, wp_lo - window + 1) : 0;
+  const int keyA = 8 * (r16 >> 2) + (r16 & 3);
+  const int kchunks = dk >> 3, vchunks = dv >> 3;
+  for (int tile = 0; tile < nsink + nmain; ++tile) {
+    const bool sink = tile < nsink;
+    const int kb = sink ? tile * PFW_BN : lo_min + (tile - nsink) * PFW_BN;
+    const int hi = sink ? min(ns, kb + PFW_BN) : min(p_max + 1, kb + PFW_BN);
+    __syncthreads();                         // the previous tile's fragments were read
+    for (int e = threadIdx.x; e < PFW_BN * kchunks; e += 256) {
+      const int ks = e / kchunks, c = e - ks * kchunks;
+      u32x4 val = u32x4{0u, 0u, 0u, 0u};
+      const int j = kb + ks;
+      if (j < hi) {
+        int b = bt[j / bs];
+        if (b < 0 || b >= num_blocks) b = 0;
+        val = *reinterpret_cast<const u32x4*>(
+            k_cache + ((int64_t)(b * G + g) * bs + (j % bs)) * dk + 8 * c);
+      }
+      *reinterpret_cast<u32x4*>(Ks + ks * kst + 8 * c) = val;
+    }
+    for (int e = threadIdx.x; e < PFW_BN * vchunks; e += 256) {
+      const int ks = e & (PFW_BN - 1), c = e >> 6;      // a wave's lanes: consecutive keys
+      Pack8<T> val;
+      val.u = u32x4{0u, 0u, 0u, 0u};
+      const int j = kb + ks;
+      if (j < hi) {
+        int b = bt[j / bs];
+        if (b < 0 || b >= num_blocks) b = 0;
+        val.u = *reinterpret_cast<const u32x4*>(
+            v_cache + ((int64_t)(b * G + g) * bs + (j % bs)) * dv + 8 * c);
+      }
+#pragma unroll
+      for (int e2 = 0; e2 < 8; ++e2) Vt[(8 * c + e2) * vst + ks] = val.h[e2];
+    }
+    __syncthreads();
+    if (16 * wave >= rows) continue;                       // no rows in this wave
+    // nothing of this tile is visible to the wave's rows (kept first tokens can sit in a
+    // main tile when the earliest window starts before them)
+    if (kb > wp_hi || (!sink && hi <= w_lo && kb >= keep_first)) continue;
+    // ---- S^T tiles j = 0..3: keys 32 (j >> 1) + keyA + 4 (j & 1)
+    f32x4 s[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const T* krow = Ks + ((j >> 1) * 32 + keyA + 4 * (j & 1)) * kst + 8 * qd;
+      f32x4 a = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s2 = 0; s2 < KSM; ++s2) {
+        if (s2 < nks) {
+          Pack8<T> fr;
+          fr.u = *reinterpret_cast<const u32x4*>(krow + 32 * s2);
+          a = mfma16x16x32(fr.v, qf[s2], a);
+        }
+      }
+      s[j] = a;
+    }
+    // ---- visibility and online softmax (query = lane & 15)
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = kb + (j >> 1) * 32 + 8 * qd + 4 * (j & 1) + i;
+        const bool vis = rowok && key < hi && key <= qpos &&
+                         (window <= 0 || qpos - key < window || key < keep_first);
+        s[j][i] = vis ? s[j][i] * scale : -INFINITY;
+        tmax = fmaxf(tmax, s[j][i]);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float mn = fmaxf(m, tmax);
+    const float alpha = m == -INFINITY ? 0.f : __expf(m - mn);
+    m = mn;
+    l *= alpha;
+    V8 phi[2], plo[2];
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      Pack8<T> ph, pl;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pa = s[2 * kk][i] == -INFINITY ? 0.f : __expf(s[2 * kk][i] - mn);
+        const float pb2 = s[2 * kk + 1][i] == -INFINITY ? 0.f : __expf(s[2 * kk + 1][i] - mn);
+        l += pa + pb2;
+        ph.h[i] = from_f<T>(pa);
+        ph.h[4 + i] = from_f<T>(pb2);
+        pl.h[i] = from_f<T>(pa - to_f(ph.h[i]));
+        pl.h[4 + i] = from_f<T>(pb2 - to_f(ph.h[4 + i]));
+      }
+      phi[kk] = ph.v;
+      plo[kk] = pl.v;
+    }
+    // ---- O^T += V^T . P^T
+#pragma unroll
+    for (int t2 = 0; t2 < DTM; ++t2) {
+      if (t2 < ndt) {
+        f32x4 acc = o[t2] * alpha;
+        const T* vrow = Vt + (16 * t2 + r16) * vst + 8 * qd;
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          Pack8<T> fr;
+          fr.u = *reinterpret_cast<const u32x4*>(vrow + 32 * kk);
+          acc = mfma16x16x32(fr.v, phi[kk], acc);
+          acc = mfma16x16x32(fr.v, plo[kk], acc);
+        }
+        o[t2] = acc;
+      }
+    }
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (rowok) {
+    const float gt = gate != nullptr ? gate[(int64_t)(q0 + myrow) * H + h] : 1.f;
+    const float inv = l > 0.f ? gt / l : 0.f;
+    T* orow = out + ((int64_t)(q0 + myrow) * H + h) * dv;
+#pragma unroll
+    for (int t2 = 0; t2 < DTM; ++t2) {
+      if (t2 < ndt) {
+        Pack4<T> w4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w4.h[i] = from_f<T>(o[t2][i] * inv);
+        *reinterpret_cast<u32x2*>(orow + 16 * t2 + 4 * qd) = w4.u;
+      }
+    }
+  }
+}
+
 }  // namespace
 
 #define KGC_DISPATCH_T(dtype, ...)                          \
@@ -178,12 +562,104 @@ void launch_window_attention(int dtype, void* out, const void* q, const void* k_
                              const int* pbt, const int* ctx_lens, const int* dbt, int bt_stride,
                              int P, int Tp, int T_, int H, int G, int dk, int dv, int bs,
                              int num_blocks, float scale, int window, int keep_first,
-                             const float* gate, hipStream_t s) {
-  if (T_ <= 0) return;
+                             const float* gate, int kinds, hipStream_t s) {
+  if (T_ <= 0 || !kinds) return;
   const size_t lds = (size_t)(dk + 128) * sizeof(float);
   KGC_DISPATCH_T(dtype, window_attention_kernel<T><<<dim3(T_, H), 64, lds, s>>>(
       (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache, qsl, seq_lens, pbt, ctx_lens,
-      dbt, bt_stride, P, Tp, H, G, dk, dv, bs, num_blocks, scale, window, keep_first, gate));
+      dbt, bt_stride, P, Tp, H, G, dk, dv, bs, num_blocks, scale, window, keep_first, gate,
+      kinds));
+}
+
+// decode rows on the 8-wave kernel: needs 16-byte key rows (dk % 8 == 0), even dv <= 512
+bool window_decode_ok(int dk, int dv, int qpg) {
+  (void)qpg;
+  return dk % 8 == 0 && dv % 2 == 0 && dv <= 128 * DEC_UMAX;
+}
+
+template <typename T>
+static void decode_dispatch(T* out, const T* q, const T* kc, const T* vc, const int* ctx_lens,
+                            const int* dbt, int bt_stride, int Tp, int D, int H, int G, int dk,
+                            int dv, int bs, int num_blocks, float scale, int window,
+                            int keep_first, const float* gate, hipStream_t s) {
+  const int qpg = H / G;
+  const int QH = qpg >= 8 ? 8 : qpg >= 3 ? 4 : qpg;      // heads per workgroup: 1, 2, 4, 8
+  const dim3 grid(D, G, (qpg + QH - 1) / QH);
+  const size_t lds = sizeof(float) * ((size_t)QH * dk + DEC_WAVES * QH * 64 + DEC_WAVES * 64 +
+                                      2 * DEC_WAVES * QH + (size_t)QH * dv);
+#define KGC_DEC(N)                                                                           \
+  window_decode_kernel<T, N><<<grid, 64 * DEC_WAVES, lds, s>>>(                              \
+      out, q, kc, vc, ctx_lens, dbt, bt_stride, Tp, H, G, dk, dv, bs, num_blocks, scale,     \
+      window, keep_first, gate)
+  if (QH == 8) KGC_DEC(8);
+  else if (QH == 4) KGC_DEC(4);
+  else if (QH == 2) KGC_DEC(2);
+  else KGC_DEC(1);
+#undef KGC_DEC
+}
+
+size_t window_decode_lds(int dk, int dv, int qpg) {
+  const int QH = qpg >= 8 ? 8 : qpg >= 3 ? 4 : qpg;
+  return sizeof(float) * ((size_t)QH * dk + DEC_WAVES * QH * 64 + DEC_WAVES * 64 +
+                          2 * DEC_WAVES * QH + (size_t)QH * dv);
+}
+
+void launch_window_decode(int dtype, void* out, const void* q, const void* k_cache,
+                          const void* v_cache, const int* ctx_lens, const int* dbt,
+                          int bt_stride, int Tp, int D, int H, int G, int dk, int dv, int bs,
+                          int num_blocks, float scale, int window, int keep_first,
+                          const float* gate, hipStream_t s) {
+  if (D <= 0) return;
+  KGC_DISPATCH_T(dtype, decode_dispatch<T>((T*)out, (const T*)q, (const T*)k_cache,
+                                           (const T*)v_cache, ctx_lens, dbt, bt_stride, Tp, D, H,
+                                           G, dk, dv, bs, num_blocks, scale, window, keep_first,
+                                           gate, s));
+}
+
+size_t window_prefill_mfma_lds(int dk, int dv) {
+  return 2 * ((size_t)PFW_BN * (dk + PFW_KPAD) + (size_t)dv * (PFW_BN + PFW_VPAD));
+}
+
+// the matrix-core prefill path: 16-bit activations, dk a multiple of 32 (<= 256), dv a
+// multiple of 16 (<= 256), both tiles within 64 KB of LDS
+bool window_prefill_mfma_ok(int dtype, int dk, int dv) {
+  return (dtype == DT_BF16 || dtype == DT_F16) && dk % 32 == 0 && dk <= 256 && dv % 16 == 0 &&
+         dv <= 256 && window_prefill_mfma_lds(dk, dv) <= 64 * 1024;
+}
+
+template <typename T>
+static void prefill_dispatch(T* out, const T* q, const T* kc, const T* vc, const int* qsl,
+                             const int* seq_lens, const int* pbt, int bt_stride,
+                             const int* work_seq, const int* work_blk, int n_work, int blk_rows,
+                             int H, int G, int dk, int dv, int bs, int num_blocks, float scale,
+                             int window, int keep_first, const float* gate, hipStream_t s) {
+  const dim3 grid(n_work * (blk_rows / PFW_BM), H);
+  const size_t lds = window_prefill_mfma_lds(dk, dv);
+#define KGC_PF(K, D)                                                                          \
+  window_prefill_mfma_kernel<T, K, D><<<grid, 256, lds, s>>>(                                 \
+      out, q, kc, vc, qsl, seq_lens, pbt, bt_stride, work_seq, work_blk, blk_rows, H, G, dk,  \
+      dv, bs, num_blocks, scale, window, keep_first, gate)
+  if (dk <= 128 && dv <= 128) KGC_PF(4, 8);
+  else KGC_PF(8, 16);
+#undef KGC_PF
+}
+
+void launch_window_prefill_mfma(int dtype, void* out, const void* q, const void* k_cache,
+                                const void* v_cache, const int* qsl, const int* seq_lens,
+                                const int* pbt, int bt_stride, const int* work_seq,
+                                const int* work_blk, int n_work, int blk_rows, int H, int G,
+                                int dk, int dv, int bs, int num_blocks, float scale, int window,
+                                int keep_first, const float* gate, hipStream_t s) {
+  if (n_work <= 0) return;
+  if (dtype == DT_BF16)
+    prefill_dispatch<bf16>((bf16*)out, (const bf16*)q, (const bf16*)k_cache,
+                           (const bf16*)v_cache, qsl, seq_lens, pbt, bt_stride, work_seq,
+                           work_blk, n_work, blk_rows, H, G, dk, dv, bs, num_blocks, scale,
+                           window, keep_first, gate, s);
+  else
+    prefill_dispatch<f16>((f16*)out, (const f16*)q, (const f16*)k_cache, (const f16*)v_cache,
+                          qsl, seq_lens, pbt, bt_stride, work_seq, work_blk, n_work, blk_rows, H,
+                          G, dk, dv, bs, num_blocks, scale, window, keep_first, gate, s);
 }
 
 }  // namespace kgc

@@ -273,7 +273,23 @@ void launch_window_attention(int dtype, void* out, const void* q, const void* k_
                              const int* pbt, const int* ctx_lens, const int* dbt, int bt_stride,
                              int P, int Tp, int T, int H, int G, int dk, int dv, int bs,
                              int num_blocks, float scale, int window, int keep_first,
-                             const float* gate, hipStream_t s);
+                             const float* gate, int kinds, hipStream_t s);
+// `kinds` above: bit 0 = run the prefill rows, bit 1 = run the decode rows (the simple kernel
+// covers whatever the two kernels below do not take)
+bool window_decode_ok(int dk, int dv, int qpg);
+size_t window_decode_lds(int dk, int dv, int qpg);
+void launch_window_decode(int dtype, void* out, const void* q, const void* k_cache,
+                          const void* v_cache, const int* ctx_lens, const int* dbt,
+                          int bt_stride, int Tp, int D, int H, int G, int dk, int dv, int bs,
+                          int num_blocks, float scale, int window, int keep_first,
+                          const float* gate, hipStream_t s);
+bool window_prefill_mfma_ok(int dtype, int dk, int dv);
+void launch_window_prefill_mfma(int dtype, void* out, const void* q, const void* k_cache,
+                                const void* v_cache, const int* qsl, const int* seq_lens,
+                                const int* pbt, int bt_stride, const int* work_seq,
+                                const int* work_blk, int n_work, int blk_rows, int H, int G,
+                                int dk, int dv, int bs, int num_blocks, float scale, int window,
+                                int keep_first, const float* gate, hipStream_t s);
 int mlstm_scan_max_dim();
 void launch_mlstm_scan(int dtype, float* out, const void* qkvg, int64_t stride,
                        const float* gates, float* S, float* nst, float* mst, const int* qsl,

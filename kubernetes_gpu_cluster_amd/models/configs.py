@@ -202,6 +202,43 @@ PRESETS: dict[str, ModelConfig] = {
                                 top_k_experts=2),
 }
 
+def _hybrid(name: str, width: int, pattern: str, att: dict, rec: dict, ff: int, vocab: int = 32000,
+            groups: int = 1) -> ModelConfig:
+    """A Dilavik-architecture preset: ``pattern`` is one letter per layer ("m": mLSTM,
+    "a": windowed attention); every layer has a dense feed-forward of ``ff``."""
+    specs = tuple(
+        MixerSpec("attention", att["heads"], att["dim"], att["vdim"], kv_heads=att["kv"],
+                  scale=att["dim"] ** -0.5, rot_dims=att["rot"], rot_base=att.get("base", 1e4),
+                  window=WindowSpec(att["window"], att["keep"]), head_gate=True, ff=ff)
+        if c == "a" else
+        MixerSpec("mlstm", rec["heads"], rec["dim"], rec["vdim"], gate_cap=rec.get("cap", 15.0), ff=ff)
+        for c in pattern)
+    return ModelConfig(name, "dilavik", len(specs), width, att["heads"], att["kv"], att["dim"], ff,
+                       vocab, max_position=8192, layer_specs=specs, norm_groups=groups,
+                       embed_scale=width ** 0.5, bos_token_id=1, eos_token_id=2)
+
+
+# Benchmark pairs of equal width, depth, head layout and (to ~5 %) parameter count: a hybrid
+# and the Llama-style decoder closest to it (bench.py --mode compare).  The hybrid's dense
+# two-matrix feed-forward is 1.5 x the gated one's intermediate size.
+PRESETS.update({
+    "dilavik-w2048": _hybrid("dilavik-w2048", 2048, "maam" * 3,
+                             dict(heads=16, kv=4, dim=128, vdim=128, rot=64, window=1024, keep=4),
+                             dict(heads=4, dim=256, vdim=512), ff=8256),
+    "llama-w2048": ModelConfig("llama-w2048", "llama", 12, 2048, 16, 4, 128, 5504, 32000,
+                               max_position=8192, rope_theta=10000.0),
+    "dilavik-w4096": _hybrid("dilavik-w4096", 4096, "maam" * 2,
+                             dict(heads=32, kv=8, dim=128, vdim=128, rot=64, window=2048, keep=4),
+                             dict(heads=8, dim=256, vdim=512), ff=21504, groups=2),
+    "llama-w4096": ModelConfig("llama-w4096", "llama", 8, 4096, 32, 8, 128, 14336, 32000,
+                               max_position=8192, rope_theta=500000.0),
+    # tests / CPU plumbing
+    "tiny-dilavik": _hybrid("tiny-dilavik", 128, "maam",
+                            dict(heads=4, kv=2, dim=32, vdim=16, rot=16, window=24, keep=2),
+                            dict(heads=2, dim=16, vdim=32), ff=192, vocab=1024, groups=2),
+})
+
+
 # HF repo basenames (lower-cased) -> preset
 _ALIASES = {
     "meta-llama-3-8b": "llama-3-8b", "meta-llama-3-8b-instruct": "llama-3-8b",

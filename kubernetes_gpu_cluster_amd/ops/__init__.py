@@ -703,6 +703,13 @@ def _row_tables(meta, T: int) -> torch.Tensor:
     return torch.cat(rows, 0)[:T]
 
 
+def window_attention_fast() -> bool:
+    """KGC_WINDOW_ATTN=simple runs every row on the one-wave-per-(row, head) kernel; by
+    default prefill chunks take the MFMA tile kernel (16-bit activations, head sizes it
+    covers) and decode rows the 8-wave kernel, the one-wave kernel taking what is left."""
+    return os.environ.get("KGC_WINDOW_ATTN", "fast") != "simple"
+
+
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                      positions: torch.Tensor, meta, scale: float, window: int, keep_first: int,
                      gate: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -719,11 +726,18 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
         return ref.window_attention(q, k_cache, v_cache, pos, _row_tables(meta, T), scale,
                                     window, keep_first, gate)
     out = torch.empty(T, H * dv, dtype=q.dtype, device=q.device)
+    ws, wb = getattr(meta, "work_seq", None), getattr(meta, "work_mblk", None)
+    if meta.num_prefills and ws is None:
+        qsl = meta.query_start_loc.tolist()
+        a, b = prefill_work_list([qsl[i + 1] - qsl[i] for i in range(meta.num_prefills)],
+                                 meta.prefill_seq_lens.tolist())
+        ws = torch.tensor(a, dtype=torch.int32, device=q.device)
+        wb = torch.tensor(b, dtype=torch.int32, device=q.device)
     _k().window_attention(out, q, k_cache, v_cache, meta.query_start_loc,
                           meta.prefill_seq_lens, meta.prefill_block_tables,
-                          meta.decode_ctx_lens, meta.decode_block_tables,
+                          meta.decode_ctx_lens, meta.decode_block_tables, ws, wb,
                           meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens,
-                          scale, window, keep_first, gate)
+                          scale, window, keep_first, gate, window_attention_fast())
     return out
 
 

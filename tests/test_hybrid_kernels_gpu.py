@@ -163,3 +163,35 @@ def test_mlstm_scan(gpu, dt, H, d, dv):
     torch.testing.assert_close(got.cpu(), want, rtol=2e-4, atol=2e-4)
     for a, b in zip(st_g, st_r):
         torch.testing.assert_close(a.cpu(), b, rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("path", ["fast", "simple"])
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("H,G,dk,dv,window,keep", [(8, 2, 96, 64, 70, 5), (4, 1, 128, 128, 150, 3),
+                                                   (4, 2, 64, 32, 0, 0), (2, 1, 160, 96, 64, 70),
+                                                   (3, 3, 32, 16, 1, 0), (6, 1, 64, 48, 129, 1)])
+def test_window_attention_long_chunks(gpu, dt, path, H, G, dk, dv, window, keep, monkeypatch):
+    """Chunks that span several 64-key tiles and 64-row blocks, continue long contexts and
+    start mid-page, next to decode rows (one of them the first token of its sequence): the
+    MFMA tile kernel and the 8-wave decode kernel (and, with KGC_WINDOW_ATTN=simple, the
+    one-wave kernel alone) against the fp32 reference."""
+    monkeypatch.setenv("KGC_WINDOW_ATTN", path)
+    torch.manual_seed(5)
+    bs = 8
+    P_q, P_sl, D_ctx = [200, 77, 130], [300, 77, 513], [400, 65, 1]
+    lens = P_sl + D_ctx
+    mb = max(lens) // bs + 1
+    nb = len(lens) * mb + 1
+    tables = (torch.randperm(nb - 1)[: len(lens) * mb].view(len(lens), mb) + 1).to(torch.int32)
+    kc = (torch.randn(nb, G, bs, dk) * 0.7).to(dt)
+    vc = torch.randn(nb, G, bs, dv).to(dt)
+    m = _meta(P_q, P_sl, D_ctx, tables)
+    T = sum(P_q) + len(D_ctx)
+    q = torch.randn(T, H, dk).to(dt)
+    pos = torch.cat([torch.arange(sl - ql, sl) for ql, sl in zip(P_q, P_sl)] +
+                    [torch.tensor([c - 1 for c in D_ctx])])
+    gate = torch.rand(T, H)
+    want = ops.window_attention(q, kc, vc, pos, m, 0.13, window, keep, gate)
+    got = ops.window_attention(q.to(gpu), kc.to(gpu), vc.to(gpu), pos.to(gpu), _to(m, gpu), 0.13,
+                               window, keep, gate.to(gpu))
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
