@@ -9,11 +9,13 @@
 // decode row is a chunk of one token).
 //
 // grid (step sequences, heads, ceil(dv / 64)), 256 threads.  A workgroup owns 64 value
-// columns of one head's S: lane = column, wave w holds rows w, w + 4, ... in registers for
-// the whole chunk, so S is read and written once per step.  Every wave keeps the whole n
-// (lane l: n[l], n[l + 64], ...) and computes the denominator itself; the numerator's four
-// row partials meet in LDS.  q / k of token t + 1 are fetched into registers while token t
-// is computed and parked in a second LDS buffer before the token's single barrier.
+// columns of one head's S: lane = column, wave w holds a contiguous quarter of the rows in
+// registers for the whole chunk, so S is read and written once per step.  Every wave keeps
+// the whole n (lane l: n[l], n[l + 64], ...) and computes the denominator itself.  Tokens
+// go in blocks of 8: their q | k, value columns and gates are staged in LDS (the next
+// block's loads are issued before the current block is computed and parked in registers),
+// each wave walks the block without a barrier, leaving its row partials of the numerators
+// in LDS, and the four partials of each token are summed after the block's barrier.
 #include "common.h"
 #include "launch.h"
 
@@ -24,7 +26,9 @@ namespace {
 constexpr int NT = 256;
 constexpr int NW = NT / 64;
 
-// RMAX: rows of S per thread (d <= 4 * RMAX); NU: n entries per lane (d <= 64 * NU)
+constexpr int TB = 8;      // tokens per block
+
+// RMAX: rows of S per thread (d <= 4 * RMAX, RMAX a multiple of 4); NU: n entries per lane
 template <typename T, int RMAX>
 __global__ __launch_bounds__(NT) void mlstm_scan_kernel(
     float* __restrict__ out, const T* __restrict__ qkvg, int64_t stride,
@@ -33,9 +37,15 @@ __global__ __launch_bounds__(NT) void mlstm_scan_kernel(
     const int* __restrict__ ctx_lens, const int* __restrict__ slots, int P, int Tp, int H,
     int d, int dv, int num_slots) {
   constexpr int NU = (4 * RMAX + 63) / 64;
+  constexpr int NQK = (TB * 2 * 4 * RMAX + NT - 1) / NT;   // staged q | k values per thread
+  constexpr int NV = TB * 64 / NT;                          // staged v values per thread
   extern __shared__ float lds[];
-  float* qk = lds;                       // [2][2 * d]: q | k of a token, double-buffered
-  float* part = lds + 4 * d;             // [2][NW][64]
+  const int dp = 4 * RMAX;                // padded row count: q | k rows are [2 * dp] in LDS
+  float* qk = lds;                        // [TB][2 * dp]: q (scaled) | k, zero beyond d
+  float* vv = qk + TB * 2 * dp;           // [TB][64]
+  float* gg = vv + TB * 64;               // [TB][2]: log input gate, log forget gate
+  float* dens = gg + TB * 2;              // [TB]
+  float* part = dens + TB;                // [TB][NW][64]
   const int s = blockIdx.x, h = blockIdx.y;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int col = blockIdx.z * 64 + lane;
@@ -62,9 +72,10 @@ __global__ __launch_bounds__(NT) void mlstm_scan_kernel(
   float Sr[RMAX], nr[NU];
   float m = 0.f;
   const bool fresh = pos0 == 0;
+  const int rbase = wave * RMAX;          // this wave's rows: rbase .. rbase + RMAX - 1
 #pragma unroll
   for (int i = 0; i < RMAX; ++i) {
-    const int r = wave + NW * i;
+    const int r = rbase + i;
     Sr[i] = (!fresh && r < d && colok) ? Ss[(int64_t)r * dv + col] : 0.f;
   }
 #pragma unroll
@@ -75,78 +86,100 @@ __global__ __launch_bounds__(NT) void mlstm_scan_kernel(
   if (!fresh) m = *ms;
   const float qscale = 1.f / sqrtf((float)d);
   const int koff = H * d, voff = 2 * H * d;
-  // prologue: token 0's q | k into LDS buffer 0
-  {
-    const T* row = qkvg + (int64_t)start * stride;
-    for (int e = threadIdx.x; e < 2 * d; e += NT)
-      qk[e] = e < d ? to_f(row[h * d + e]) * qscale : to_f(row[koff + h * d + (e - d)]);
-  }
+  float pqk[NQK], pv[NV], pg = 0.f;
+
+  // global -> registers for the block of tokens starting at t0 (zeros beyond the chunk / d)
+  auto fetch = [&](int t0) {
+#pragma unroll
+    for (int j = 0; j < NQK; ++j) {
+      const int e = threadIdx.x + NT * j;
+      const int tb = e / (2 * dp), c = e - tb * 2 * dp;
+      float val = 0.f;
+      if (tb < TB && t0 + tb < len) {
+        const T* row = qkvg + (int64_t)(start + t0 + tb) * stride;
+        if (c < dp) { if (c < d) val = to_f(row[h * d + c]) * qscale; }
+        else if (c - dp < d) val = to_f(row[koff + h * d + (c - dp)]);
+      }
+      pqk[j] = val;
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) {
+      const int e = threadIdx.x + NT * j, tb = e >> 6, c = blockIdx.z * 64 + (e & 63);
+      pv[j] = (t0 + tb < len && c < dv)
+                  ? to_f(qkvg[(int64_t)(start + t0 + tb) * stride + voff + h * dv + c]) : 0.f;
+    }
+    if (threadIdx.x < 2 * TB) {
+      const int tb = threadIdx.x >> 1, which = threadIdx.x & 1;
+      pg = t0 + tb < len ? gates[(int64_t)(start + t0 + tb) * 2 * H + which * H + h] : 0.f;
+    }
+  };
+  auto park = [&]() {
+#pragma unroll
+    for (int j = 0; j < NQK; ++j) {
+      const int e = threadIdx.x + NT * j;
+      if (e < TB * 2 * dp) qk[e] = pqk[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NV; ++j) vv[threadIdx.x + NT * j] = pv[j];
+    if (threadIdx.x < 2 * TB) gg[threadIdx.x] = pg;
+  };
+
+  fetch(0);
+  park();
   __syncthreads();
-  for (int t = 0; t < len; ++t) {
-    const int64_t tok = start + t;
-    const T* row = qkvg + tok * stride;
-    const float* cur = qk + (t & 1) * 2 * d;
-    float* nxt = qk + ((t + 1) & 1) * 2 * d;
-    // fetch the next token's q | k (held in registers across this token's math)
-    float pre[(2 * 4 * RMAX + NT - 1) / NT];
-    if (t + 1 < len) {
-      const T* nrow = row + stride;
+  for (int t0 = 0; t0 < len; t0 += TB) {
+    const int nb = min(TB, len - t0);
+    if (t0 + TB < len) fetch(t0 + TB);           // in flight while this block is computed
+    for (int tb = 0; tb < nb; ++tb) {
+      const float* cq = qk + tb * 2 * dp;
+      const float* ck = cq + dp;
+      const float ig = gg[2 * tb], fg = gg[2 * tb + 1];
+      const float mn = fmaxf(fg + m, ig);
+      const float fa = expf(fg + m - mn), ia = expf(ig - mn);
+      m = mn;
+      float nq = 0.f;
 #pragma unroll
-      for (int j = 0; j < (2 * 4 * RMAX + NT - 1) / NT; ++j) {
-        const int e = threadIdx.x + NT * j;
-        pre[j] = e < 2 * d ? (e < d ? to_f(nrow[h * d + e]) * qscale
-                                    : to_f(nrow[koff + h * d + (e - d)])) : 0.f;
+      for (int u = 0; u < NU; ++u) {
+        const int r = lane + 64 * u;            // r < dp always; rows beyond d hold zeros
+        nr[u] = fa * nr[u] + ia * ck[r];
+        nq += nr[u] * cq[r];
+      }
+      nq = wave_sum(nq);
+      if (wave == 0 && lane == 0) dens[tb] = fmaxf(fabsf(nq), expf(-mn)) + 1e-6f;
+      const float iv = ia * vv[tb * 64 + lane];
+      float n0 = 0.f, n1 = 0.f, n2 = 0.f, n3 = 0.f;       // independent chains
+#pragma unroll
+      for (int i = 0; i < RMAX; i += 4) {
+        const float4 k4 = *reinterpret_cast<const float4*>(ck + rbase + i);
+        const float4 q4 = *reinterpret_cast<const float4*>(cq + rbase + i);
+        Sr[i] = fa * Sr[i] + k4.x * iv;
+        Sr[i + 1] = fa * Sr[i + 1] + k4.y * iv;
+        Sr[i + 2] = fa * Sr[i + 2] + k4.z * iv;
+        Sr[i + 3] = fa * Sr[i + 3] + k4.w * iv;
+        n0 += Sr[i] * q4.x;
+        n1 += Sr[i + 1] * q4.y;
+        n2 += Sr[i + 2] * q4.z;
+        n3 += Sr[i + 3] * q4.w;
+      }
+      const float num = (n0 + n1) + (n2 + n3);
+      part[(tb * NW + wave) * 64 + lane] = num;
+    }
+    __syncthreads();                              // partials complete; qk / vv / gg consumed
+    for (int tb = wave; tb < nb; tb += NW) {
+      if (colok) {
+        float tot = 0.f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) tot += part[(tb * NW + w) * 64 + lane];
+        out[((int64_t)(start + t0 + tb) * H + h) * dv + col] = tot / dens[tb];
       }
     }
-    const float ig = gates[tok * 2 * H + h], fg = gates[tok * 2 * H + H + h];
-    const float v = colok ? to_f(row[voff + h * dv + col]) : 0.f;
-    const float mn = fmaxf(fg + m, ig);
-    const float fa = expf(fg + m - mn), ia = expf(ig - mn);
-    m = mn;
-    // normaliser and denominator (every wave, whole n)
-    float nq = 0.f;
-#pragma unroll
-    for (int u = 0; u < NU; ++u) {
-      const int r = lane + 64 * u;
-      if (r < d) {
-        nr[u] = fa * nr[u] + ia * cur[d + r];
-        nq += nr[u] * cur[r];
-      }
-    }
-    nq = wave_sum(nq);
-    const float den = fmaxf(fabsf(nq), expf(-mn)) + 1e-6f;
-    // memory update and this wave's rows of the numerator
-    const float iv = ia * v;
-    float num = 0.f;
-#pragma unroll
-    for (int i = 0; i < RMAX; ++i) {
-      const int r = wave + NW * i;
-      if (r < d) {
-        Sr[i] = fa * Sr[i] + cur[d + r] * iv;
-        num += Sr[i] * cur[r];
-      }
-    }
-    float* pp = part + (t & 1) * NW * 64;
-    pp[wave * 64 + lane] = num;
-    if (t + 1 < len) {
-#pragma unroll
-      for (int j = 0; j < (2 * 4 * RMAX + NT - 1) / NT; ++j) {
-        const int e = threadIdx.x + NT * j;
-        if (e < 2 * d) nxt[e] = pre[j];
-      }
-    }
-    __syncthreads();
-    if (wave == 0 && colok) {
-      float tot = 0.f;
-#pragma unroll
-      for (int w = 0; w < NW; ++w) tot += pp[w * 64 + lane];
-      out[(tok * H + h) * dv + col] = tot / den;
-    }
+    if (t0 + TB < len) park();
+    __syncthreads();                              // next block staged; partials consumed
   }
   // the step's final state back to the slot
 #pragma unroll
   for (int i = 0; i < RMAX; ++i) {
-    const int r = wave + NW * i;
+    const int r = rbase + i;
     if (r < d && colok) Ss[(int64_t)r * dv + col] = Sr[i];
   }
   if (blockIdx.z == 0 && wave == 0) {
@@ -159,17 +192,20 @@ __global__ __launch_bounds__(NT) void mlstm_scan_kernel(
   }
 }
 
+static size_t scan_lds(int rmax) {
+  return sizeof(float) * (size_t)(TB * 2 * 4 * rmax + TB * 64 + TB * 2 + TB + TB * NW * 64);
+}
+
 template <typename T>
 void scan_dispatch(float* out, const T* qkvg, int64_t stride, const float* gates, float* S,
                    float* nst, float* mst, const int* qsl, const int* seq_lens,
                    const int* ctx_lens, const int* slots, int P, int D, int Tp, int H, int d,
                    int dv, int num_slots, hipStream_t s) {
   const dim3 grid(P + D, H, (dv + 63) / 64);
-  const size_t lds = (size_t)(4 * d + 2 * NW * 64) * sizeof(float);
 #define KGC_SCAN(R)                                                                          \
-  mlstm_scan_kernel<T, R><<<grid, NT, lds, s>>>(out, qkvg, stride, gates, S, nst, mst, qsl, \
-                                                seq_lens, ctx_lens, slots, P, Tp, H, d, dv, \
-                                                num_slots)
+  mlstm_scan_kernel<T, R><<<grid, NT, scan_lds(R), s>>>(out, qkvg, stride, gates, S, nst, mst, \
+                                                        qsl, seq_lens, ctx_lens, slots, P, Tp, \
+                                                        H, d, dv, num_slots)
   if (d <= 64) KGC_SCAN(16);
   else if (d <= 128) KGC_SCAN(32);
   else if (d <= 256) KGC_SCAN(64);

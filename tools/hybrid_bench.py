@@ -1,0 +1,184 @@
+"""Microbenchmarks of the hybrid-decoder kernels beside the Llama-path kernel each one is
+closest to, at the layer shapes of the dilavik-w2048 / llama-w2048 presets.
+
+    python tools/hybrid_bench.py [--reps 20] > profiles/hybrid_kernels.jsonl
+
+One JSON line per kernel and shape: microseconds per call (events around `reps` calls) and
+the bytes or FLOPs the call has to move or do at least, as GB/s or TFLOP/s.  Prefill shape:
+32 chunks of 512 tokens (16384 rows); decode shapes: 64 and 256 rows at context 544."""
+import argparse
+import json
+import types
+
+import torch
+
+from kubernetes_gpu_cluster_amd import ops
+from kubernetes_gpu_cluster_amd.ops import reference as ref
+
+DEV = torch.device("cuda")
+BF = torch.bfloat16
+
+
+def timed(fn, reps):
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / reps
+
+
+def emit(name, shape, us, gbytes=None, tflop=None, like=None):
+    r = {"kernel": name, "shape": shape, "us": round(us, 1)}
+    if gbytes is not None:
+        r["GB_s"] = round(gbytes / us * 1e6, 0)
+    if tflop is not None:
+        r["TFLOP_s"] = round(tflop / us * 1e6, 1)
+    if like:
+        r["like"] = like
+    print(json.dumps(r), flush=True)
+
+
+def meta(P_q, P_sl, D_ctx, bs, dev, slots=None):
+    m = types.SimpleNamespace()
+    P, D = len(P_q), len(D_ctx)
+    lens = P_sl + D_ctx
+    mb = max(lens) // bs + 1
+    tables = (torch.arange(len(lens) * mb, dtype=torch.int32).view(len(lens), mb) + 1).to(dev)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)   # noqa: E731
+    qsl = [0]
+    for q in P_q:
+        qsl.append(qsl[-1] + q)
+    m.num_prefills, m.num_decodes, m.num_prefill_tokens = P, D, qsl[-1]
+    m.query_start_loc = i32(qsl) if P else None
+    m.prefill_seq_lens = i32(P_sl) if P else None
+    m.prefill_block_tables = tables[:P].contiguous() if P else None
+    m.decode_ctx_lens = i32(D_ctx) if D else None
+    m.decode_block_tables = tables[P:].contiguous() if D else None
+    m.state_slots = i32(slots) if slots is not None else None
+    if P:
+        ws, wb = ops.prefill_work_list(P_q, P_sl)
+        m.work_seq, m.work_mblk = i32(ws), i32(wb)
+    return m, tables, len(lens) * mb + 1
+
+
+def attention(reps):
+    H, G, d, bs, W, keep = 16, 4, 128, 32, 1024, 4
+    for name, P_q, P_sl, D_ctx in (("prefill 32x512", [512] * 32, [512] * 32, []),
+                                   ("prefill 8x2048", [2048] * 8, [2048] * 8, []),
+                                   ("decode 64 @544", [], [], [544] * 64),
+                                   ("decode 256 @544", [], [], [544] * 256)):
+        m, tables, nb = meta(P_q, P_sl, D_ctx, bs, DEV)
+        T = sum(P_q) + len(D_ctx)
+        q = torch.randn(T, H, d, device=DEV, dtype=BF)
+        kc = torch.randn(nb, G, bs, d, device=DEV, dtype=BF)
+        vc = torch.randn(nb, G, bs, d, device=DEV, dtype=BF)
+        gate = torch.rand(T, H, device=DEV)
+        pos = torch.zeros(T, dtype=torch.int64, device=DEV)
+        us = timed(lambda: ops.window_attention(q, kc, vc, pos, m, 0.09, W, keep, gate), reps)
+        # visible (query, key) pairs -> 2 * pairs * (dk + dv) FLOPs per head; decode: K/V bytes
+        pairs = sum(sum(min(p + 1, W) + max(0, min(keep, p + 1 - W)) for p in range(sl - ql, sl))
+                    for ql, sl in zip(P_q, P_sl))
+        if P_q:
+            emit("window_attention (MFMA tile)", name, us, tflop=2 * pairs * 2 * d * H / 1e12)
+            kc2 = kc
+            vc2 = torch.randn(nb, G, bs // 8, d, 8, device=DEV, dtype=BF)
+            us2 = timed(lambda: ops.prefill_attention(q, kc2, vc2, m.prefill_block_tables,
+                                                      m.query_start_loc, m.prefill_seq_lens, 0.09,
+                                                      m.work_seq, m.work_mblk), reps)
+            full = sum(sum(p + 1 for p in range(sl - ql, sl)) for ql, sl in zip(P_q, P_sl))
+            emit("prefill_attention (K2, causal)", name, us2, tflop=2 * full * 2 * d * H / 1e12,
+                 like="window_attention")
+        else:
+            gb = sum(min(c, W + keep) for c in D_ctx) * G * 2 * d * 2 / 1e9
+            emit("window_attention (8-wave decode)", name, us, gbytes=gb)
+            vc2 = torch.randn(nb, G, bs // 8, d, 8, device=DEV, dtype=BF)
+            z = ops.decode_grid_z(len(D_ctx), G, max(D_ctx))
+            ws = ops.decode_partials(len(D_ctx), H, d, tables.shape[1], bs, DEV)
+            us2 = timed(lambda: ops.paged_attention_decode(q, kc, vc2, m.decode_block_tables,
+                                                           m.decode_ctx_lens, 0.09, ws, z), reps)
+            emit("paged_attention_decode (K1)", name, us2, gbytes=sum(D_ctx) * G * 2 * d * 2 / 1e9,
+                 like="window_attention")
+
+
+def recurrent(reps):
+    H, d, dv = 4, 256, 512
+    N = 2 * H * d + 2 * H * dv
+    for name, P_q, D_ctx in (("prefill 32x512", [512] * 32, []), ("decode 64", [], [100] * 64),
+                             ("decode 256", [], [100] * 256)):
+        n = len(P_q) + len(D_ctx)
+        m, _, _ = meta(P_q, list(P_q), D_ctx, 32, DEV, slots=list(range(n)))
+        T = sum(P_q) + len(D_ctx)
+        qkvg = torch.randn(T, N, device=DEV, dtype=BF)
+        gates = torch.cat([torch.randn(T, H, device=DEV), -torch.rand(T, H, device=DEV)], 1)
+        st = (torch.zeros(n, H, d, dv, device=DEV), torch.zeros(n, H, d, device=DEV),
+              torch.zeros(n, H, device=DEV))
+        us = timed(lambda: ops.mlstm_scan(qkvg, gates, st, m, H, d, dv), reps)
+        # per token and head: S update + read-out = 4 d dv FLOPs; per step: state read + write
+        emit("mlstm_scan", name, us, gbytes=2 * n * H * d * dv * 4 / 1e9,
+             tflop=4 * T * H * d * dv / 1e12)
+
+
+def rows(reps):
+    W, L = 2048, 12
+    for T in (16384, 64, 256):
+        x = torch.randn(T, W, device=DEV)
+        y = torch.randn(T, W, device=DEV, dtype=BF)
+        w = torch.ones(W, device=DEV)
+        hist = torch.randn(L + 1, T, W, device=DEV)
+        coef = torch.randn(L + 1, device=DEV)
+        us = timed(lambda: ops.group_rms_norm(x, w, 1, 1e-5, BF, add=y), reps)
+        emit("group_rms_norm(add)", f"{T}x{W}", us, gbytes=T * W * (4 + 4 + 2 + 2) / 1e9)
+        xb, rb, wb = y.clone(), y.clone(), torch.ones(W, device=DEV, dtype=BF)
+        us = timed(lambda: ops.fused_add_rms_norm(xb, rb, wb, 1e-5), reps)
+        emit("fused_add_rms_norm (K4)", f"{T}x{W}", us, gbytes=T * W * 8 / 1e9,
+             like="group_rms_norm(add)")
+        for layer in (0, 5, 11):
+            us = timed(lambda: ops.depth_mix_norm(x, hist, layer, y, coef, w, 1, 1e-5, BF), reps)
+            emit(f"depth_mix_norm layer {layer}", f"{T}x{W}", us,
+                 gbytes=T * W * (4 * (layer + 1) + 4 + 4 + 4 + 2 + 2) / 1e9)
+        z = torch.randn(T, 8256, device=DEV, dtype=BF)
+        ab = torch.tensor([0.7, 1.2], device=DEV)
+        us = timed(lambda: ops.xielu(z, ab), reps)
+        emit("xielu", f"{T}x8256", us, gbytes=T * 8256 * 4 / 1e9)
+        gu = torch.randn(T, 2 * 5504, device=DEV, dtype=BF)
+        us = timed(lambda: ops.silu_mul(gu), reps)
+        emit("silu_mul (K7)", f"{T}x5504", us, gbytes=T * 5504 * 6 / 1e9, like="xielu")
+        h = torch.randn(T, W, device=DEV, dtype=BF)
+        wg = torch.randn(16, W, device=DEV, dtype=BF)
+        us = timed(lambda: ops.gate_proj(h, wg, None, ops.GATE_SIGMOID), reps)
+        emit("gate_proj N=16", f"{T}x{W}", us, gbytes=T * W * 2 / 1e9)
+        o = torch.randn(T, 2048, device=DEV)
+        g = torch.randn(T, 2048, device=DEV, dtype=BF)
+        us = timed(lambda: ops.head_norm_gate(o, g, w, 4, 1e-5, BF), reps)
+        emit("head_norm_gate", f"{T}x2048", us, gbytes=T * 2048 * 8 / 1e9)
+        # rotary + cache store
+        H, G, d, bs = 16, 4, 128, 32
+        nb = T // bs + 2
+        qkv = torch.randn(T, (H + 2 * G) * d, device=DEV, dtype=BF)
+        kc = torch.zeros(nb, G, bs, d, device=DEV, dtype=BF)
+        vc = torch.zeros(nb, G, bs, d, device=DEV, dtype=BF)
+        pos = (torch.arange(T, device=DEV) % 512).to(torch.int64)
+        slots = torch.arange(T, device=DEV, dtype=torch.int64) + bs
+        table = ref.rope_table(64, 4096, 1e4).to(DEV)
+        us = timed(lambda: ops.rope_kv_store(qkv, pos, table, kc, vc, slots, H, G, d, d), reps)
+        emit("rope_kv_store", f"{T} rows", us, gbytes=T * (H + 2 * G) * d * 4 / 1e9)
+        cs = ref.rope_cos_sin_cache(d, 4096, 1e4).to(DEV)
+        vc2 = torch.zeros(nb, G, bs // 8, d, 8, device=DEV, dtype=BF)
+        us = timed(lambda: ops.rope_kv_write(qkv, pos, cs, kc, vc2, slots, H, G, d), reps)
+        emit("rope_kv_write (K3)", f"{T} rows", us, gbytes=T * (H + 2 * G) * d * 4 / 1e9,
+             like="rope_kv_store")
+
+
+if __name__ == "__main__":
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--only", default="attention,recurrent,rows")
+    a = ap.parse_args()
+    ops.load_extension(strict=True)
+    for part in a.only.split(","):
+        {"attention": attention, "recurrent": recurrent, "rows": rows}[part](a.reps)
