@@ -169,6 +169,35 @@ __device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
   }
 }
 
+// the same 8 elements kept as loaded (4 registers for 16-bit types) until they are used
+template <typename T> struct Raw8 { u32x4 u; };
+template <> struct Raw8<float> { float4 a, b; };
+
+template <typename T>
+__device__ __forceinline__ Raw8<T> load8raw(const T* p) {
+  Raw8<T> r;
+  if constexpr (std::is_same_v<T, float>) {
+    r.a = *reinterpret_cast<const float4*>(p);
+    r.b = *reinterpret_cast<const float4*>(p + 4);
+  } else {
+    r.u = *reinterpret_cast<const u32x4*>(p);
+  }
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ void cvt8(const Raw8<T>& r, float (&v)[8]) {
+  if constexpr (std::is_same_v<T, float>) {
+    v[0] = r.a.x; v[1] = r.a.y; v[2] = r.a.z; v[3] = r.a.w;
+    v[4] = r.b.x; v[5] = r.b.y; v[6] = r.b.z; v[7] = r.b.w;
+  } else {
+    Pack8<T> t;
+    t.u = r.u;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = to_f(t.h[e]);
+  }
+}
+
 template <typename T>
 __device__ __forceinline__ void load2(const T* p, float& a, float& b) {
   if constexpr (std::is_same_v<T, float>) {
@@ -235,6 +264,8 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
   }
   float* pw = pb + wave * QH * 64;
   int* ow = ob + wave * 64;
+  const int lpr = dv >> 3;                 // lanes per value row in the 16-byte path
+  const bool vrow = (dv & 7) == 0 && lpr <= 64 && (lpr & (lpr - 1)) == 0;
   for (int chunk = wave; chunk < nchunks; chunk += DEC_WAVES) {
     const int idx = chunk * 64 + lane;
     const bool ok = idx < total;
@@ -276,6 +307,36 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     const int cnt = min(64, total - chunk * 64);
+    if (vrow) {
+      // lpr lanes cover a value row with 16-byte loads; the 64 / lpr lane groups take
+      // every (64 / lpr)-th key of the chunk and are summed once, after the last chunk
+#pragma unroll
+      for (int h = 0; h < QH; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[h][e >> 1][e & 1] *= alpha[h];
+      const int ci = lane & (lpr - 1), cg = lane / lpr, kg = 64 / lpr;
+      constexpr int VB = std::is_same_v<T, float> ? 4 : 8;    // rows in flight per lane
+      for (int j0 = cg; j0 < cnt; j0 += VB * kg) {
+        Raw8<T> raw[VB];
+#pragma unroll
+        for (int b = 0; b < VB; ++b) {
+          const int jj = min(j0 + b * kg, cnt - 1);            // clamped: weight 0 below
+          raw[b] = load8raw(v_cache + (int64_t)ow[jj] * dv + 8 * ci);
+        }
+#pragma unroll
+        for (int b = 0; b < VB; ++b) {
+          const int jj = j0 + b * kg;
+          float v8[8];
+          cvt8(raw[b], v8);
+#pragma unroll
+          for (int h = 0; h < QH; ++h) {
+            const float p = jj < cnt ? pw[h * 64 + min(jj, 63)] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[h][e >> 1][e & 1] += p * v8[e];
+          }
+        }
+      }
+    } else {
 #pragma unroll
     for (int u = 0; u < DEC_UMAX; ++u) {
       const int c0 = 2 * lane + 128 * u;
@@ -303,6 +364,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
         }
       }
     }
+    }
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
@@ -321,8 +383,23 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
     for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, mm[w * QH + h]);
     f[h] = m[h] == -INFINITY ? 0.f : expf(m[h] - M);
   }
+  if (vrow) {
+    for (int off = lpr; off < 64; off <<= 1)
+#pragma unroll
+      for (int h = 0; h < QH; ++h)
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          acc[h][e >> 1][e & 1] += __shfl_xor(acc[h][e >> 1][e & 1], off, 64);
+  }
   for (int w = 0; w < DEC_WAVES; ++w) {
-    if (wave == w && nchunks > w) {
+    if (vrow) {
+      if (wave == w && nchunks > w && lane < lpr) {
+#pragma unroll
+        for (int h = 0; h < QH; ++h)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) accs[h * dv + 8 * lane + e] += acc[h][e >> 1][e & 1] * f[h];
+      }
+    } else if (wave == w && nchunks > w) {
 #pragma unroll
       for (int u = 0; u < DEC_UMAX; ++u) {
         const int c0 = 2 * lane + 128 * u;
@@ -365,7 +442,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
 constexpr int PFW_BM = 64, PFW_BN = 64, PFW_KPAD = 8, PFW_VPAD = 8;
 
 template <typename T, int KSM, int DTM>
-__global__ __launch_bounds__(256) void window_prefill_mfma_kernel(
+__global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const int* __restrict__ pbt, int bt_stride, const int* __restrict__ work_seq,
@@ -414,36 +491,40 @@ __global__ __launch_bounds__(256) void window_prefill_mfma_kernel(
   const int w_lo = window > 0 ? max(0, wp_lo - window + 1) : 0;
   const int keyA = 8 * (r16 >> 2) + (r16 & 3);
   const int kchunks = dk >> 3, vchunks = dv >> 3;
+  const int bs_shift = (bs & (bs - 1)) == 0 ? __builtin_ctz(bs) : -1;
+  auto page_row = [&](int key) -> int64_t {
+    const int pg = bs_shift >= 0 ? key >> bs_shift : key / bs;
+    const int in = bs_shift >= 0 ? key & (bs - 1) : key - pg * bs;
+    int bl = bt[pg];
+    if (bl < 0 || bl >= num_blocks) bl = 0;
+    return (int64_t)(bl * G + g) * bs + in;
+  };
+  const int sr = threadIdx.x >> 4, sc = threadIdx.x & 15;     // K staging: 16 lanes per key row
   for (int tile = 0; tile < nsink + nmain; ++tile) {
     const bool sink = tile < nsink;
     const int kb = sink ? tile * PFW_BN : lo_min + (tile - nsink) * PFW_BN;
     const int hi = sink ? min(ns, kb + PFW_BN) : min(p_max + 1, kb + PFW_BN);
     __syncthreads();                         // the previous tile's fragments were read
-    for (int e = threadIdx.x; e < PFW_BN * kchunks; e += 256) {
-      const int ks = e / kchunks, c = e - ks * kchunks;
-      u32x4 val = u32x4{0u, 0u, 0u, 0u};
-      const int j = kb + ks;
-      if (j < hi) {
-        int b = bt[j / bs];
-        if (b < 0 || b >= num_blocks) b = 0;
-        val = *reinterpret_cast<const u32x4*>(
-            k_cache + ((int64_t)(b * G + g) * bs + (j % bs)) * dk + 8 * c);
-      }
-      *reinterpret_cast<u32x4*>(Ks + ks * kst + 8 * c) = val;
-    }
-    for (int e = threadIdx.x; e < PFW_BN * vchunks; e += 256) {
-      const int ks = e & (PFW_BN - 1), c = e >> 6;      // a wave's lanes: consecutive keys
-      Pack8<T> val;
-      val.u = u32x4{0u, 0u, 0u, 0u};
-      const int j = kb + ks;
-      if (j < hi) {
-        int b = bt[j / bs];
-        if (b < 0 || b >= num_blocks) b = 0;
-        val.u = *reinterpret_cast<const u32x4*>(
-            v_cache + ((int64_t)(b * G + g) * bs + (j % bs)) * dv + 8 * c);
-      }
 #pragma unroll
-      for (int e2 = 0; e2 < 8; ++e2) Vt[(8 * c + e2) * vst + ks] = val.h[e2];
+    for (int kq = 0; kq < 4; ++kq) {
+      const int ks = sr + 16 * kq, key = kb + ks;
+      const T* src = key < hi ? k_cache + page_row(key) * dk : nullptr;
+      for (int c = sc; c < kchunks; c += 16) {
+        u32x4 val = u32x4{0u, 0u, 0u, 0u};
+        if (src != nullptr) val = *reinterpret_cast<const u32x4*>(src + 8 * c);
+        *reinterpret_cast<u32x4*>(Ks + ks * kst + 8 * c) = val;
+      }
+    }
+    {
+      const int ks = threadIdx.x & (PFW_BN - 1), key = kb + ks;   // a wave's lanes: consecutive keys
+      const T* src = key < hi ? v_cache + page_row(key) * dv : nullptr;
+      for (int c = threadIdx.x >> 6; c < vchunks; c += 4) {
+        Pack8<T> val;
+        val.u = u32x4{0u, 0u, 0u, 0u};
+        if (src != nullptr) val.u = *reinterpret_cast<const u32x4*>(src + 8 * c);
+#pragma unroll
+        for (int e2 = 0; e2 < 8; ++e2) Vt[(8 * c + e2) * vst + ks] = val.h[e2];
+      }
     }
     __syncthreads();
     if (16 * wave >= rows) continue;                       // no rows in this wave
@@ -466,18 +547,32 @@ __global__ __launch_bounds__(256) void window_prefill_mfma_kernel(
       }
       s[j] = a;
     }
-    // ---- visibility and online softmax (query = lane & 15)
+    // ---- visibility and online softmax (query = lane & 15).  A tile whose 64 keys are
+    // all valid, not after the wave's first row and inside the window of its last row is
+    // seen in full by every row of the wave: no per-element test.
+    const bool full = hi == kb + PFW_BN && kb + PFW_BN - 1 <= wp_lo &&
+                      (window <= 0 || wp_hi - kb < window) && wp_lo + 15 == wp_hi;
     float tmax = -INFINITY;
+    if (full) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = kb + (j >> 1) * 32 + 8 * qd + 4 * (j & 1) + i;
-        const bool vis = rowok && key < hi && key <= qpos &&
-                         (window <= 0 || qpos - key < window || key < keep_first);
-        s[j][i] = vis ? s[j][i] * scale : -INFINITY;
-        tmax = fmaxf(tmax, s[j][i]);
-      }
+        for (int i = 0; i < 4; ++i) {
+          s[j][i] *= scale;
+          tmax = fmaxf(tmax, s[j][i]);
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int key = kb + (j >> 1) * 32 + 8 * qd + 4 * (j & 1) + i;
+          const bool vis = rowok && key < hi && key <= qpos &&
+                           (window <= 0 || qpos - key < window || key < keep_first);
+          s[j][i] = vis ? s[j][i] * scale : -INFINITY;
+          tmax = fmaxf(tmax, s[j][i]);
+        }
+    }
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
     const float mn = fmaxf(m, tmax);
