@@ -143,6 +143,56 @@ __global__ __launch_bounds__(NT) void gate_proj_kernel(
   }
 }
 
+// Many rows: a workgroup keeps 8 rows of w in registers (thread t: columns t, t + 256, ...)
+// and walks rows bx, bx + gridDim.x, ...; per row each thread multiplies its columns of h
+// into 8 partial sums, which meet through wave shuffles and a double-buffered LDS table.
+template <typename T, int CPT>
+__global__ __launch_bounds__(NT) void gate_proj_rows_kernel(
+    float* __restrict__ out, const T* __restrict__ h, const T* __restrict__ w,
+    const float* __restrict__ bias, int rows, int W, int N, int kind_a, int kind_b, int split,
+    float cap) {
+  constexpr int NB = 8;
+  __shared__ float red[2][NT / 64][NB];
+  const int n0 = blockIdx.y * NB;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float wr[NB][CPT];
+#pragma unroll
+  for (int n = 0; n < NB; ++n)
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      const int c = threadIdx.x + NT * j;
+      wr[n][j] = (n0 + n < N && c < W) ? to_f(w[(int64_t)(n0 + n) * W + c]) : 0.f;
+    }
+  int it = 0;
+  for (int row = blockIdx.x; row < rows; row += gridDim.x, ++it) {
+    const T* hr = h + (int64_t)row * W;
+    float acc[NB];
+#pragma unroll
+    for (int n = 0; n < NB; ++n) acc[n] = 0.f;
+#pragma unroll
+    for (int j = 0; j < CPT; ++j) {
+      const int c = threadIdx.x + NT * j;
+      const float hv = c < W ? to_f(hr[c]) : 0.f;
+#pragma unroll
+      for (int n = 0; n < NB; ++n) acc[n] += hv * wr[n][j];
+    }
+#pragma unroll
+    for (int n = 0; n < NB; ++n) {
+      const float t = wave_sum(acc[n]);
+      if (lane == 0) red[it & 1][wave][n] = t;
+    }
+    __syncthreads();
+    if (threadIdx.x < NB && n0 + threadIdx.x < N) {
+      const int n = n0 + threadIdx.x;
+      float t = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < NT / 64; ++wv) t += red[it & 1][wv][threadIdx.x];
+      if (bias != nullptr) t += bias[n];
+      out[(int64_t)row * N + n] = gate_act(t, n < split ? kind_a : kind_b, cap);
+    }
+  }
+}
+
 }  // namespace
 
 #define KGC_DISPATCH_T(dtype, ...)                          \
@@ -185,6 +235,18 @@ void launch_gate_proj(int dtype, float* out, const void* h, const void* w, const
                       int rows, int W, int N, int kind_a, int kind_b, int split, float cap,
                       hipStream_t s) {
   if (rows <= 0) return;
+  if (rows >= 1024 && W <= 16 * NT) {
+    // enough rows to amortise holding w in registers: 8 outputs per workgroup column
+    const dim3 grid(1024, (N + 7) / 8);
+#define KGC_GP(C)                                                                      \
+  KGC_DISPATCH_T(dtype, gate_proj_rows_kernel<T, C><<<grid, NT, 0, s>>>(               \
+      out, (const T*)h, (const T*)w, bias, rows, W, N, kind_a, kind_b, split, cap))
+    if (W <= 4 * NT) KGC_GP(4);
+    else if (W <= 8 * NT) KGC_GP(8);
+    else KGC_GP(16);
+#undef KGC_GP
+    return;
+  }
   const size_t lds = (size_t)W * sizeof(float);
   KGC_DISPATCH_T(dtype, gate_proj_kernel<T><<<rows, NT, lds, s>>>(
       out, (const T*)h, (const T*)w, bias, W, N, kind_a, kind_b, split, cap));

@@ -122,6 +122,19 @@ def models(tmp_path_factory):
 _engines = {}
 
 
+@pytest.fixture(scope="module", autouse=True)
+def _release_engines():
+    """Engines are shared by the tests of this module and released after the last one."""
+    yield
+    for eng in _engines.values():
+        eng.shutdown()
+    _engines.clear()
+    import gc
+    gc.collect()
+    if torch.cuda.is_available():
+        torch.cuda.empty_cache()
+
+
 def engine(models, name, device, dtype, pages=24, page=8, seqs=4, **kw):
     if device == "cuda" and not torch.cuda.is_available():
         pytest.skip("no GPU")

@@ -195,3 +195,17 @@ def test_window_attention_long_chunks(gpu, dt, path, H, G, dk, dv, window, keep,
     got = ops.window_attention(q.to(gpu), kc.to(gpu), vc.to(gpu), pos.to(gpu), _to(m, gpu), 0.13,
                                window, keep, gate.to(gpu))
     torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
+
+
+@pytest.mark.parametrize("dt", DT)
+@pytest.mark.parametrize("rows,W,N", [(1500, 320, 10), (2048, 1536, 8), (1100, 2304, 19)])
+def test_gate_proj_many_rows(gpu, dt, rows, W, N):
+    """The row-blocked kernel (weights held in registers, >= 1024 rows)."""
+    torch.manual_seed(6)
+    h = torch.randn(rows, W).to(dt)
+    w = (torch.randn(N, W) * 0.1).to(dt)
+    b = torch.randn(N)
+    want = ref.gate_proj(h, w, b, ops.GATE_CAP_TANH, ops.GATE_LOGSIG_CAP_TANH, N // 2, 9.0)
+    got = ops.gate_proj(h.to(gpu), w.to(gpu), b.to(gpu), ops.GATE_CAP_TANH,
+                        ops.GATE_LOGSIG_CAP_TANH, N // 2, 9.0)
+    torch.testing.assert_close(got.cpu(), want, rtol=2e-4, atol=2e-4)
