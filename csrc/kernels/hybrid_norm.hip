@@ -119,8 +119,9 @@ __device__ __forceinline__ float gate_act(float y, int kind, float cap) {
   return fminf(y, 0.f) - log1pf(expf(-fabsf(y)));
 }
 
-// one workgroup per row; the row of h sits in LDS as fp32, each wave takes outputs
-// n = wave, wave + 4, ...
+// Few rows: grid (rows, ceil(N / 4)); the row of h sits in LDS as fp32 and each of the four
+// waves computes one output, eight independent 64-column strips at a time so that the
+// weight loads of a strip group are all in flight together.
 template <typename T>
 __global__ __launch_bounds__(NT) void gate_proj_kernel(
     float* __restrict__ out, const T* __restrict__ h, const T* __restrict__ w,
@@ -131,15 +132,27 @@ __global__ __launch_bounds__(NT) void gate_proj_kernel(
   for (int c = threadIdx.x; c < W; c += NT) hrow[c] = to_f(hr[c]);
   __syncthreads();
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  for (int n = wave; n < N; n += NT / 64) {
-    const T* wr = w + (int64_t)n * W;
-    float acc = 0.f;
-    for (int c = lane; c < W; c += 64) acc += hrow[c] * to_f(wr[c]);
-    acc = wave_sum(acc);
-    if (lane == 0) {
-      if (bias != nullptr) acc += bias[n];
-      out[row * N + n] = gate_act(acc, n < split ? kind_a : kind_b, cap);
+  const int n = blockIdx.y * (NT / 64) + wave;
+  if (n >= N) return;
+  const T* wr = w + (int64_t)n * W;
+  float acc = 0.f;
+  for (int c0 = lane; c0 < W; c0 += 64 * 8) {
+    float wv[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int c = c0 + 64 * u;
+      wv[u] = c < W ? to_f(wr[c]) : 0.f;
     }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int c = c0 + 64 * u;
+      if (c < W) acc += hrow[c] * wv[u];
+    }
+  }
+  acc = wave_sum(acc);
+  if (lane == 0) {
+    if (bias != nullptr) acc += bias[n];
+    out[row * N + n] = gate_act(acc, n < split ? kind_a : kind_b, cap);
   }
 }
 
@@ -248,7 +261,8 @@ void launch_gate_proj(int dtype, float* out, const void* h, const void* w, const
     return;
   }
   const size_t lds = (size_t)W * sizeof(float);
-  KGC_DISPATCH_T(dtype, gate_proj_kernel<T><<<rows, NT, lds, s>>>(
+  const dim3 grid(rows, (N + NT / 64 - 1) / (NT / 64));
+  KGC_DISPATCH_T(dtype, gate_proj_kernel<T><<<grid, NT, lds, s>>>(
       out, (const T*)h, (const T*)w, bias, W, N, kind_a, kind_b, split, cap));
 }
 
