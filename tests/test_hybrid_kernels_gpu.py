@@ -18,7 +18,7 @@ def _tol(dt):
 
 
 @pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("W,G", [(320, 2), (384, 3), (1024, 1)])
+@pytest.mark.parametrize("W,G", [(352, 2), (384, 3), (1024, 1)])
 def test_group_norm_and_add(gpu, dt, W, G):
     torch.manual_seed(0)
     x = torch.randn(37, W) * 3
@@ -59,8 +59,8 @@ def test_xielu_gate_proj_head_norm(gpu, dt):
     ab = torch.tensor([0.7, 1.3])
     torch.testing.assert_close(ops.xielu(z.to(gpu), ab.to(gpu)).cpu().float(),
                                ref.xielu(z, ab).float(), **_tol(dt))
-    h = torch.randn(13, 320).to(dt)
-    w = (torch.randn(10, 320) * 0.2).to(dt)
+    h = torch.randn(13, 288).to(dt)
+    w = (torch.randn(10, 288) * 0.2).to(dt)
     b = torch.randn(10)
     want = ref.gate_proj(h, w, b, ops.GATE_CAP_TANH, ops.GATE_LOGSIG_CAP_TANH, 5, 15.0)
     got = ops.gate_proj(h.to(gpu), w.to(gpu), b.to(gpu), ops.GATE_CAP_TANH,
@@ -167,7 +167,7 @@ def test_mlstm_scan(gpu, dt, H, d, dv):
 
 @pytest.mark.parametrize("path", ["fast", "simple"])
 @pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("H,G,dk,dv,window,keep", [(8, 2, 96, 64, 70, 5), (4, 1, 128, 128, 150, 3),
+@pytest.mark.parametrize("H,G,dk,dv,window,keep", [(4, 2, 96, 64, 70, 5), (4, 1, 128, 128, 150, 3),
                                                    (4, 2, 64, 32, 0, 0), (2, 1, 160, 96, 64, 70),
                                                    (3, 3, 32, 16, 1, 0), (6, 1, 64, 48, 129, 1)])
 def test_window_attention_long_chunks(gpu, dt, path, H, G, dk, dv, window, keep, monkeypatch):
@@ -198,7 +198,7 @@ def test_window_attention_long_chunks(gpu, dt, path, H, G, dk, dv, window, keep,
 
 
 @pytest.mark.parametrize("dt", DT)
-@pytest.mark.parametrize("rows,W,N", [(1500, 320, 10), (2048, 1536, 8), (1100, 2304, 19)])
+@pytest.mark.parametrize("rows,W,N", [(1500, 288, 10), (2048, 1536, 8), (1100, 2304, 19)])
 def test_gate_proj_many_rows(gpu, dt, rows, W, N):
     """The row-blocked kernel (weights held in registers, >= 1024 rows)."""
     torch.manual_seed(6)
