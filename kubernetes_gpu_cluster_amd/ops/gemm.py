@@ -254,6 +254,10 @@ def skinny_gemm(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    if x.dtype == torch.float32:
+        # the tuned kernels are 16-bit; an fp32 engine (true fp32 GEMMs) in a process that
+        # also tuned a 16-bit one must not pick up its (M, N, K) plan
+        return F.linear(x, w, bias)
     if x.is_cuda and x.dim() == 2 and x.shape[0] <= SKINNY_MAX_M and _plan:
         cfg = _plan.get((x.shape[0], w.shape[0], w.shape[1]))
         if cfg is not None and x.stride(1) == 1:

@@ -58,6 +58,15 @@ PLAIN = config([att(heads=2, kv=2, dim=16, vdim=16, rot=16, size=6, keep=0, ff=0
                width=64, vocab=96, groups=1, scale=1.0)
 
 
+# head sizes the matrix-core prefill kernel and the 16-byte decode paths take (key sizes of
+# 64 and 96, value sizes of 32 and 48), two attention layers of different shape, a wider mLSTM
+WIDE = config([att(heads=4, kv=2, dim=64, vdim=32, rot=32, size=40, keep=3, scale=0.15, ff=96),
+               mls(heads=2, dim=72, vdim=40, cap=12.0, ff=0),
+               att(heads=6, kv=1, dim=96, vdim=48, rot=64, base=500.0, size=70, keep=0, scale=0.12,
+                   ff=0)],
+              width=128, vocab=200, groups=4, scale=3.0)
+
+
 def write_model(path, cfg, seed):
     """Random bf16 weights in the checkpoint's naming; returns them as float64 arrays."""
     from safetensors.torch import save_file
@@ -113,7 +122,7 @@ def write_model(path, cfg, seed):
 def models(tmp_path_factory):
     root = tmp_path_factory.mktemp("dilavik")
     out = {}
-    for name, cfg, seed in (("mixed", MIXED, 11), ("plain", PLAIN, 12)):
+    for name, cfg, seed in (("mixed", MIXED, 11), ("plain", PLAIN, 12), ("wide", WIDE, 13)):
         d = str(root / name)
         out[name] = (d, cfg, write_model(d, cfg, seed))
     return out
@@ -187,12 +196,12 @@ def run_alone(rp, rid, toks, cuts):
 
 # ---------------------------------------------------------------- whole prompts, decode, portions
 @pytest.mark.parametrize("device,dtype", DEVICES)
-@pytest.mark.parametrize("name", ["mixed", "plain"])
+@pytest.mark.parametrize("name", ["mixed", "plain", "wide"])
 def test_whole_prompt_matches_oracle(models, name, device, dtype):
     _, cfg, wts = models[name]
     eng = engine(models, name, device, dtype)
     rp = TraceReplayer(eng)
-    toks = tokens_for(cfg, 61, 1)
+    toks = tokens_for(cfg, 150 if name == "wide" else 61, 1)
     want = oracle.forward(toks, cfg, wts)
     got = run_alone(rp, "w", toks, [len(toks)])
     assert close(got, want, dtype)
@@ -203,14 +212,16 @@ def test_whole_prompt_matches_oracle(models, name, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", DEVICES)
-@pytest.mark.parametrize("name", ["mixed", "plain"])
+@pytest.mark.parametrize("name", ["mixed", "plain", "wide"])
 def test_prefill_then_token_by_token(models, name, device, dtype):
     _, cfg, wts = models[name]
     eng = engine(models, name, device, dtype)
     rp = TraceReplayer(eng)
-    toks = tokens_for(cfg, 70, 2)
+    toks = tokens_for(cfg, 130 if name == "wide" else 70, 2)
     want = oracle.forward(toks, cfg, wts)
-    got = run_alone(rp, "d", toks, [20, 1])        # 50 decoded tokens: every window passes
+    if name == "wide":                             # portions across 64-row blocks and key tiles
+        assert close(run_alone(rp, "c", toks, [70, 3, 45, 2, 1]), want, dtype)
+    got = run_alone(rp, "d", toks, [20, 1])        # decoded tokens: every window passes
     assert close(got, want, dtype)
     got = run_alone(rp, "e", toks, [1])            # decoding from the very first token
     assert close(got, want, dtype)
