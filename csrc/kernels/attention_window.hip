@@ -219,11 +219,11 @@ __device__ __forceinline__ void load2(const T* p, float& a, float& b) {
 // two value columns and walks the chunk's 64 value rows, again once for all heads.  Every
 // wave carries its own online-softmax state per head; the eight states merge in LDS in
 // wave order (deterministic).  Scores, weights and sums are fp32.
-constexpr int DEC_WAVES = 8;
+constexpr int DEC_WAVES = 8;          // waves per workgroup (4 when the grid is large)
 constexpr int DEC_UMAX = 4;          // value columns per lane: 2 * DEC_UMAX * 64 >= dv
 
-template <typename T, int QH>
-__global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
+template <typename T, int QH, int NWV>
+__global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ ctx_lens, const int* __restrict__ dbt,
     int bt_stride, int Tp, int H, int G, int dk, int dv, int bs, int num_blocks, float scale,
@@ -234,21 +234,21 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
   const int t = Tp + dd, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   float* qs = lds;                                    // [QH][dk]
   float* pb = qs + QH * dk;                           // [waves][QH][64]
-  int* ob = (int*)(pb + DEC_WAVES * QH * 64);         // [waves][64]
-  float* mm = (float*)(ob + DEC_WAVES * 64);          // [waves][QH]
-  float* ml = mm + DEC_WAVES * QH;                    // [waves][QH]
-  float* accs = ml + DEC_WAVES * QH;                  // [QH][dv]
+  int* ob = (int*)(pb + NWV * QH * 64);         // [waves][64]
+  float* mm = (float*)(ob + NWV * 64);          // [waves][QH]
+  float* ml = mm + NWV * QH;                    // [waves][QH]
+  float* accs = ml + NWV * QH;                  // [QH][dv]
   const int h0 = g * qpg + hq0;                       // first query head of this workgroup
   const int pos = ctx_lens[dd] - 1;
   const int* bt = dbt + (int64_t)dd * bt_stride;
   if (pos < 0 || pos >= bt_stride * bs) {             // a padding row: zeros
-    for (int e = threadIdx.x; e < nh * dv; e += 64 * DEC_WAVES)
+    for (int e = threadIdx.x; e < nh * dv; e += 64 * NWV)
       out[((int64_t)t * H + h0) * dv + e] = from_f<T>(0.f);
     return;
   }
-  for (int e = threadIdx.x; e < nh * dk; e += 64 * DEC_WAVES)
+  for (int e = threadIdx.x; e < nh * dk; e += 64 * NWV)
     qs[e] = to_f(q[((int64_t)t * H + h0) * dk + e]);
-  for (int e = threadIdx.x; e < QH * dv; e += 64 * DEC_WAVES) accs[e] = 0.f;
+  for (int e = threadIdx.x; e < QH * dv; e += 64 * NWV) accs[e] = 0.f;
   __syncthreads();
   const int lo_w = window > 0 ? max(0, pos - window + 1) : 0;
   const int ns = min(keep_first, lo_w);
@@ -266,7 +266,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
   int* ow = ob + wave * 64;
   const int lpr = dv >> 3;                 // lanes per value row in the 16-byte path
   const bool vrow = (dv & 7) == 0 && lpr <= 64 && (lpr & (lpr - 1)) == 0;
-  for (int chunk = wave; chunk < nchunks; chunk += DEC_WAVES) {
+  for (int chunk = wave; chunk < nchunks; chunk += NWV) {
     const int idx = chunk * 64 + lane;
     const bool ok = idx < total;
     float sc[QH];
@@ -279,15 +279,28 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
       if (b < 0 || b >= num_blocks) b = 0;
       ro = (b * G + g) * bs + (j % bs);
       const T* kr = k_cache + (int64_t)ro * dk;
-      for (int c = 0; c < dk; c += 8) {
-        float kv[8];
-        load8(kr + c, kv);
+      constexpr int KB = 8;                       // 16-byte pieces of the key row in flight
+      for (int c0 = 0; c0 < dk; c0 += 8 * KB) {
+        Raw8<T> kraw[KB];
 #pragma unroll
-        for (int h = 0; h < QH; ++h) {
-          if (h < nh) {
-            const float* qh = qs + h * dk + c;
+        for (int b = 0; b < KB; ++b) {
+          const int c = min(c0 + 8 * b, dk - 8);  // clamped: pieces past dk are not used
+          kraw[b] = load8raw(kr + c);
+        }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) sc[h] += qh[e] * kv[e];
+        for (int b = 0; b < KB; ++b) {
+          const int c = c0 + 8 * b;
+          if (c < dk) {
+            float kv[8];
+            cvt8(kraw[b], kv);
+#pragma unroll
+            for (int h = 0; h < QH; ++h) {
+              if (h < nh) {
+                const float* qh = qs + h * dk + c;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) sc[h] += qh[e] * kv[e];
+              }
+            }
           }
         }
       }
@@ -380,7 +393,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
 #pragma unroll
   for (int h = 0; h < QH; ++h) {
     float M = -INFINITY;
-    for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, mm[w * QH + h]);
+    for (int w = 0; w < NWV; ++w) M = fmaxf(M, mm[w * QH + h]);
     f[h] = m[h] == -INFINITY ? 0.f : expf(m[h] - M);
   }
   if (vrow) {
@@ -391,7 +404,7 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
         for (int e = 0; e < 8; ++e)
           acc[h][e >> 1][e & 1] += __shfl_xor(acc[h][e >> 1][e & 1], off, 64);
   }
-  for (int w = 0; w < DEC_WAVES; ++w) {
+  for (int w = 0; w < NWV; ++w) {
     if (vrow) {
       if (wave == w && nchunks > w && lane < lpr) {
 #pragma unroll
@@ -414,11 +427,11 @@ __global__ __launch_bounds__(64 * DEC_WAVES) void window_decode_kernel(
     }
     __syncthreads();
   }
-  for (int e = threadIdx.x; e < nh * dv; e += 64 * DEC_WAVES) {
+  for (int e = threadIdx.x; e < nh * dv; e += 64 * NWV) {
     const int h = e / dv;
     float M = -INFINITY, L = 0.f;
-    for (int w = 0; w < DEC_WAVES; ++w) M = fmaxf(M, mm[w * QH + h]);
-    for (int w = 0; w < DEC_WAVES; ++w) {
+    for (int w = 0; w < NWV; ++w) M = fmaxf(M, mm[w * QH + h]);
+    for (int w = 0; w < NWV; ++w) {
       const float mw = mm[w * QH + h];
       if (mw != -INFINITY) L += ml[w * QH + h] * expf(mw - M);
     }
@@ -672,6 +685,11 @@ bool window_decode_ok(int dk, int dv, int qpg) {
   return dk % 8 == 0 && dv % 2 == 0 && dv <= 128 * DEC_UMAX;
 }
 
+static size_t decode_lds(int QH, int nwv, int dk, int dv) {
+  return sizeof(float) * ((size_t)QH * dk + (size_t)nwv * QH * 64 + nwv * 64 + 2 * nwv * QH +
+                          (size_t)QH * dv);
+}
+
 template <typename T>
 static void decode_dispatch(T* out, const T* q, const T* kc, const T* vc, const int* ctx_lens,
                             const int* dbt, int bt_stride, int Tp, int D, int H, int G, int dk,
@@ -680,23 +698,28 @@ static void decode_dispatch(T* out, const T* q, const T* kc, const T* vc, const 
   const int qpg = H / G;
   const int QH = qpg >= 8 ? 8 : qpg >= 3 ? 4 : qpg;      // heads per workgroup: 1, 2, 4, 8
   const dim3 grid(D, G, (qpg + QH - 1) / QH);
-  const size_t lds = sizeof(float) * ((size_t)QH * dk + DEC_WAVES * QH * 64 + DEC_WAVES * 64 +
-                                      2 * DEC_WAVES * QH + (size_t)QH * dv);
-#define KGC_DEC(N)                                                                           \
-  window_decode_kernel<T, N><<<grid, 64 * DEC_WAVES, lds, s>>>(                              \
+  // 8 waves split a row's keys finest (shortest chain per workgroup); once the grid holds
+  // two workgroups per CU, 4-wave workgroups let two of them overlap on a CU instead
+  const bool small = (int64_t)grid.x * grid.y * grid.z >= 512;
+#define KGC_DEC(N, W)                                                                        \
+  window_decode_kernel<T, N, W><<<grid, 64 * W, decode_lds(N, W, dk, dv), s>>>(              \
       out, q, kc, vc, ctx_lens, dbt, bt_stride, Tp, H, G, dk, dv, bs, num_blocks, scale,     \
       window, keep_first, gate)
-  if (QH == 8) KGC_DEC(8);
-  else if (QH == 4) KGC_DEC(4);
-  else if (QH == 2) KGC_DEC(2);
-  else KGC_DEC(1);
+#define KGC_DEC2(N) \
+  do {              \
+    if (small) KGC_DEC(N, 4); else KGC_DEC(N, 8); \
+  } while (0)
+  if (QH == 8) KGC_DEC2(8);
+  else if (QH == 4) KGC_DEC2(4);
+  else if (QH == 2) KGC_DEC2(2);
+  else KGC_DEC2(1);
+#undef KGC_DEC2
 #undef KGC_DEC
 }
 
 size_t window_decode_lds(int dk, int dv, int qpg) {
   const int QH = qpg >= 8 ? 8 : qpg >= 3 ? 4 : qpg;
-  return sizeof(float) * ((size_t)QH * dk + DEC_WAVES * QH * 64 + DEC_WAVES * 64 +
-                          2 * DEC_WAVES * QH + (size_t)QH * dv);
+  return decode_lds(QH, DEC_WAVES, dk, dv);
 }
 
 void launch_window_decode(int dtype, void* out, const void* q, const void* k_cache,

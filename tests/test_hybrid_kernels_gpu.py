@@ -209,3 +209,24 @@ def test_gate_proj_many_rows(gpu, dt, rows, W, N):
     got = ops.gate_proj(h.to(gpu), w.to(gpu), b.to(gpu), ops.GATE_CAP_TANH,
                         ops.GATE_LOGSIG_CAP_TANH, N // 2, 9.0)
     torch.testing.assert_close(got.cpu(), want, rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("dt", DT)
+def test_window_attention_many_decode_rows(gpu, dt):
+    """A decode batch large enough (rows x kv heads >= 512) for the 4-wave workgroups."""
+    torch.manual_seed(8)
+    H, G, dk, dv, bs, window, keep = 4, 2, 64, 32, 8, 50, 3
+    g = torch.Generator().manual_seed(9)
+    D_ctx = torch.randint(1, 200, (300,), generator=g).tolist()
+    mb = max(D_ctx) // bs + 1
+    nb = 64
+    tables = torch.randint(1, nb, (len(D_ctx), mb), generator=g).to(torch.int32)
+    kc = (torch.randn(nb, G, bs, dk) * 0.7).to(dt)
+    vc = torch.randn(nb, G, bs, dv).to(dt)
+    m = _meta([], [], D_ctx, tables)
+    q = torch.randn(len(D_ctx), H, dk).to(dt)
+    pos = torch.tensor([c - 1 for c in D_ctx])
+    want = ops.window_attention(q, kc, vc, pos, m, 0.2, window, keep, None)
+    got = ops.window_attention(q.to(gpu), kc.to(gpu), vc.to(gpu), pos.to(gpu), _to(m, gpu), 0.2,
+                               window, keep, None)
+    torch.testing.assert_close(got.cpu().float(), want.float(), **_tol(dt))
