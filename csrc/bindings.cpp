@@ -1390,7 +1390,28 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   TORCH_CHECK(q.dim() == 3 && q.is_contiguous() && act_dtype(q), "kgc.window_attention: q [T, H, dk]");
   const int64_t T = q.size(0), H = q.size(1), dk = q.size(2);
   const int64_t G = k_cache.size(1), dv = v_cache.size(3);
-  check_plain_cache(k_cache, v_cache, q, G, dk, dv);
+  int64_t krs = dk, vrs = dv;
+  if (v_cache.is_contiguous()) {
+    check_plain_cache(k_cache, v_cache, q, G, dk, dv);
+  } else {
+    // values as columns of other cache rows (a view of the key cache): same pages, same
+    // rows, its own row stride
+    TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() &&
+                k_cache.size(3) == dk && v_cache.size(0) == k_cache.size(0) &&
+                v_cache.size(1) == G && v_cache.size(2) == k_cache.size(2) &&
+                v_cache.stride(3) == 1 && v_cache.stride(1) == v_cache.size(2) * v_cache.stride(2) &&
+                v_cache.stride(0) == G * v_cache.stride(1) && dv <= v_cache.stride(2),
+                "kgc.window_attention: strided values must keep the cache's page / row order");
+    TORCH_CHECK(k_cache.scalar_type() == q.scalar_type() && v_cache.scalar_type() == q.scalar_type() &&
+                k_cache.device() == q.device() && v_cache.device() == q.device(),
+                "kgc: cache dtype / device must match the activations");
+    TORCH_CHECK(k_cache.size(0) * G * k_cache.size(2) < (int64_t(1) << 31), "kgc: cache rows exceed int32");
+    vrs = v_cache.stride(2);
+  }
+  // 16-byte row loads of the fast kernels
+  const int64_t vec = q.scalar_type() == at::kFloat ? 4 : 8;
+  const bool aligned = krs % vec == 0 && vrs % vec == 0 &&
+                       reinterpret_cast<uintptr_t>(v_cache.data_ptr()) % 16 == 0;
   TORCH_CHECK(G >= 1 && H % G == 0 && H <= 65535, "kgc.window_attention: heads");
   TORCH_CHECK(dk <= 4096 && dv <= kgc::window_attention_max_dv(), "kgc.window_attention: head sizes");
   TORCH_CHECK(out.is_contiguous() && out.numel() == T * H * dv &&
@@ -1412,7 +1433,7 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
   const int* dp = i32_ptr(dbt, D, "decode block tables");
   const int bs = (int)k_cache.size(2), nb = (int)k_cache.size(0), dt = dt_code(q);
   int rest = 3;                   // row kinds the one-wave kernel still has to run
-  if (fast && P > 0 && work_seq.has_value() && work_blk.has_value() &&
+  if (fast && aligned && P > 0 && work_seq.has_value() && work_blk.has_value() &&
       kgc::window_prefill_mfma_ok(dt, (int)dk, (int)dv)) {
     const int64_t nw = work_seq->numel();
     TORCH_CHECK(work_blk->numel() == nw && work_seq->scalar_type() == at::kInt &&
@@ -1421,24 +1442,24 @@ void window_attention(Tensor out, Tensor q, Tensor k_cache, Tensor v_cache,
     kgc::launch_window_prefill_mfma(dt, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                                     v_cache.data_ptr(), qp, sp, pp, (int)bts,
                                     work_seq->data_ptr<int>(), work_blk->data_ptr<int>(), (int)nw,
-                                    kgc::prefill_block_m(), (int)H, (int)G, (int)dk, (int)dv, bs,
-                                    nb, (float)scale, (int)window, (int)keep_first, gp, stream());
+                                    kgc::prefill_block_m(), (int)H, (int)G, (int)dk, (int)dv,
+                                    (int)krs, (int)vrs, bs, nb, (float)scale, (int)window, (int)keep_first, gp, stream());
     rest &= ~1;
   }
-  if (fast && D > 0 && kgc::window_decode_ok((int)dk, (int)dv, (int)(H / G)) &&
+  if (fast && aligned && D > 0 && kgc::window_decode_ok((int)dk, (int)dv, (int)(H / G)) &&
       kgc::window_decode_lds((int)dk, (int)dv, (int)(H / G)) <= 64 * 1024) {
     kgc::launch_window_decode(dt, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                               v_cache.data_ptr(), cp, dp, (int)bts, (int)Tp, (int)D, (int)H,
-                              (int)G, (int)dk, (int)dv, bs, nb, (float)scale, (int)window,
-                              (int)keep_first, gp, stream());
+                              (int)G, (int)dk, (int)dv, (int)krs, (int)vrs, bs, nb, (float)scale,
+                              (int)window, (int)keep_first, gp, stream());
     rest &= ~2;
   }
   if (!P) rest &= ~1;
   if (!D) rest &= ~2;
   kgc::launch_window_attention(dt, out.data_ptr(), q.data_ptr(), k_cache.data_ptr(),
                                v_cache.data_ptr(), qp, sp, pp, cp, dp, (int)bts, (int)P, (int)Tp,
-                               (int)T, (int)H, (int)G, (int)dk, (int)dv, bs, nb, (float)scale,
-                               (int)window, (int)keep_first, gp, rest, stream());
+                               (int)T, (int)H, (int)G, (int)dk, (int)dv, (int)krs, (int)vrs, bs, nb,
+                               (float)scale, (int)window, (int)keep_first, gp, rest, stream());
 }
 
 void mlstm_scan(Tensor out, Tensor qkvg, Tensor gates, Tensor S, Tensor n, Tensor m,
@@ -1470,9 +1491,260 @@ void mlstm_scan(Tensor out, Tensor qkvg, Tensor gates, Tensor S, Tensor n, Tenso
                          (int)d, (int)dv, (int)S.size(0), stream());
 }
 
+// ---- scaled residual stream, token shift, minGRU, latent attention rows, sigmoid routing --
+const float* f32_opt(const std::optional<Tensor>& t, int64_t numel, const char* name) {
+  if (!t.has_value()) return nullptr;
+  check_f32(*t, name);
+  TORCH_CHECK(t->numel() == numel, "kgc: ", name, " must have ", numel, " entries");
+  return t->data_ptr<float>();
+}
+
+void residual_norm(std::optional<Tensor> out, Tensor x, std::optional<Tensor> add,
+                   std::optional<Tensor> add_norm_w, std::optional<Tensor> w, double mult,
+                   double eps) {
+  check_f32(x, "x");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+  TORCH_CHECK(x.dim() == 2, "kgc.residual_norm: x [rows, W]");
+  const int64_t rows = x.size(0), W = x.size(1);
+  int dt = kgc::DT_F32, odt = kgc::DT_F32;
+  const void* ap = nullptr;
+  if (add.has_value()) {
+    TORCH_CHECK(add->is_cuda() && add->is_contiguous() && add->sizes() == x.sizes() &&
+                act_dtype(*add) && add->device() == x.device(), "kgc.residual_norm: add");
+    dt = dt_code(*add);
+    ap = add->data_ptr();
+  }
+  void* op = nullptr;
+  if (out.has_value()) {
+    TORCH_CHECK(out->is_cuda() && out->is_contiguous() && out->sizes() == x.sizes() &&
+                act_dtype(*out) && out->device() == x.device(), "kgc.residual_norm: out");
+    odt = dt_code(*out);
+    if (!add.has_value()) dt = odt;
+    TORCH_CHECK(odt == kgc::DT_F32 || odt == dt,
+                "kgc.residual_norm: out is fp32 or of the addend's dtype");
+    op = out->data_ptr();
+  }
+  TORCH_CHECK(!add_norm_w.has_value() || add.has_value(), "kgc.residual_norm: add_norm_w without add");
+  kgc::launch_residual_norm(dt, odt, op, x.data_ptr<float>(), ap,
+                            f32_opt(add_norm_w, W, "add_norm_w"), f32_opt(w, W, "w"),
+                            (float)mult, (int)rows, (int)W, (float)eps, stream());
+}
+
+struct StepSeqs {
+  const int *qsl, *sl, *ctx, *slots;
+};
+
+StepSeqs step_seqs(const std::optional<Tensor>& qsl, const std::optional<Tensor>& seq_lens,
+                   const std::optional<Tensor>& ctx_lens, const Tensor& slots, int64_t P,
+                   int64_t D, int64_t Tp, int64_t T) {
+  TORCH_CHECK(Tp + D == T && P >= 0 && D >= 0 && (P > 0) == (Tp > 0), "kgc: step counts");
+  return {i32_ptr(qsl, P ? P + 1 : 0, "query_start_loc"), i32_ptr(seq_lens, P, "seq_lens"),
+          i32_ptr(ctx_lens, D, "ctx_lens"), i32_ptr(slots, P + D, "state slots")};
+}
+
+void token_shift(Tensor out, Tensor h, Tensor mu, Tensor state, std::optional<Tensor> qsl,
+                 std::optional<Tensor> seq_lens, std::optional<Tensor> ctx_lens, Tensor slots,
+                 int64_t P, int64_t D, int64_t Tp) {
+  check_f32(h, "h");
+  check_f32(mu, "mu");
+  check_f32(state, "state");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
+  TORCH_CHECK(h.dim() == 2 && out.is_cuda() && out.is_contiguous() && out.sizes() == h.sizes() &&
+              act_dtype(out) && out.device() == h.device(), "kgc.token_shift: out / h [T, W]");
+  const int64_t T = h.size(0), W = h.size(1);
+  TORCH_CHECK(mu.numel() == W && state.dim() == 2 && state.size(1) == W,
+              "kgc.token_shift: mu [W], state [slots, W]");
+  const StepSeqs q = step_seqs(qsl, seq_lens, ctx_lens, slots, P, D, Tp, T);
+  kgc::launch_token_shift(dt_code(out), out.data_ptr(), h.data_ptr<float>(), mu.data_ptr<float>(),
+                          state.data_ptr<float>(), q.qsl, q.sl, q.ctx, q.slots, (int)P, (int)Tp,
+                          (int)T, (int)W, (int)state.size(0), stream());
+}
+
+void mingru_scan(Tensor out, Tensor zxg, Tensor bias, Tensor state, std::optional<Tensor> qsl,
+                 std::optional<Tensor> seq_lens, std::optional<Tensor> ctx_lens, Tensor slots,
+                 int64_t P, int64_t D, int64_t Tp, int64_t width) {
+  check_gpu(zxg, "zxg");
+  check_f32(bias, "bias");
+  check_f32(state, "state");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(zxg.device());
+  TORCH_CHECK(zxg.dim() == 2 && zxg.stride(1) == 1 && act_dtype(zxg) && width >= 1 &&
+              zxg.size(1) >= 3 * width, "kgc.mingru_scan: zxg [T, 3 width]");
+  const int64_t T = zxg.size(0);
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.dim() == 2 && out.size(0) == T &&
+              out.size(1) == width && out.scalar_type() == zxg.scalar_type() &&
+              out.device() == zxg.device(), "kgc.mingru_scan: out [T, width]");
+  TORCH_CHECK(bias.numel() == 2 * width && state.dim() == 2 && state.size(1) == width,
+              "kgc.mingru_scan: bias [2 width], state [slots, width]");
+  const StepSeqs q = step_seqs(qsl, seq_lens, ctx_lens, slots, P, D, Tp, T);
+  kgc::launch_mingru_scan(dt_code(zxg), out.data_ptr(), zxg.data_ptr(), zxg.stride(0),
+                          bias.data_ptr<float>(), state.data_ptr<float>(), q.qsl, q.sl, q.ctx,
+                          q.slots, (int)P, (int)D, (int)Tp, (int)width, (int)state.size(0),
+                          stream());
+}
+
+void latent_rope_store(Tensor q_out, Tensor proj, Tensor q_lat, Tensor positions,
+                       std::optional<Tensor> table, Tensor norm_w, double eps, Tensor cache,
+                       Tensor slots, int64_t H, int64_t d, int64_t r, int64_t rank) {
+  check_gpu(proj, "proj");
+  check_f32(norm_w, "norm_w");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
+  TORCH_CHECK(H >= 1 && d >= 0 && r >= 0 && r % 2 == 0 && rank >= 1, "kgc.latent_rope_store: sizes");
+  TORCH_CHECK(proj.dim() == 2 && proj.stride(1) == 1 && act_dtype(proj) &&
+              proj.size(1) >= H * (d + r) + rank + r, "kgc.latent_rope_store: proj [T, H (d + r) + rank + r ...]");
+  const int64_t T = proj.size(0), dk = rank + r;
+  TORCH_CHECK(q_lat.is_cuda() && q_lat.is_contiguous() && q_lat.numel() == H * T * rank &&
+              q_lat.scalar_type() == proj.scalar_type() && q_lat.device() == proj.device(),
+              "kgc.latent_rope_store: q_lat [H, T, rank]");
+  TORCH_CHECK(q_out.is_cuda() && q_out.is_contiguous() && q_out.numel() == T * H * dk &&
+              q_out.scalar_type() == proj.scalar_type() && q_out.device() == proj.device(),
+              "kgc.latent_rope_store: q_out [T, H, rank + r]");
+  TORCH_CHECK(cache.is_cuda() && cache.dim() == 4 && cache.is_contiguous() && cache.size(1) == 1 &&
+              cache.size(3) == dk && cache.scalar_type() == proj.scalar_type() &&
+              cache.device() == proj.device(), "kgc.latent_rope_store: cache [nb, 1, bs, rank + r]");
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.numel() == T &&
+              positions.is_contiguous() && slots.scalar_type() == at::kLong &&
+              slots.numel() == T && slots.is_contiguous() && positions.is_cuda() && slots.is_cuda(),
+              "kgc.latent_rope_store: positions / slots int64 [T]");
+  TORCH_CHECK(norm_w.numel() == rank, "kgc.latent_rope_store: norm_w [rank]");
+  const float* tp = nullptr;
+  int64_t rows = 0;
+  if (r > 0) {
+    TORCH_CHECK(table.has_value(), "kgc.latent_rope_store: rotary table missing");
+    check_f32(*table, "table");
+    TORCH_CHECK(table->dim() == 2 && table->size(1) == r && table->size(0) >= 1,
+                "kgc.latent_rope_store: table [max_pos, r]");
+    tp = table->data_ptr<float>();
+    rows = table->size(0);
+  }
+  kgc::launch_latent_rope_store(dt_code(proj), q_out.data_ptr(), proj.data_ptr(), proj.stride(0),
+                                q_lat.data_ptr(), positions.data_ptr<int64_t>(), tp, (int)rows,
+                                norm_w.data_ptr<float>(), (float)eps, cache.data_ptr(),
+                                slots.data_ptr<int64_t>(), cache.size(0) * cache.size(2), (int)T,
+                                (int)H, (int)d, (int)r, (int)rank, stream());
+}
+
+void gate_mul(Tensor out, Tensor o, Tensor gt) {
+  check_gpu(o, "o");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(o.device());
+  TORCH_CHECK(o.dim() == 3 && o.stride(2) == 1 && act_dtype(o), "kgc.gate_mul: o [T, H, dv]");
+  const int64_t T = o.size(0), H = o.size(1), dv = o.size(2);
+  TORCH_CHECK(gt.is_cuda() && gt.dim() == 2 && gt.size(0) == T && gt.size(1) == H * dv &&
+              gt.stride(1) == 1 && gt.scalar_type() == o.scalar_type() && gt.device() == o.device(),
+              "kgc.gate_mul: gate [T, H dv]");
+  TORCH_CHECK(out.is_cuda() && out.is_contiguous() && out.numel() == T * H * dv &&
+              out.scalar_type() == o.scalar_type() && out.device() == o.device(), "kgc.gate_mul: out");
+  kgc::launch_gate_mul(dt_code(o), out.data_ptr(), o.data_ptr(), o.stride(0), o.stride(1),
+                       gt.data_ptr(), gt.stride(0), (int)T, (int)H, (int)dv, stream());
+}
+
+void relu_sq(Tensor out, Tensor z) {
+  check_gpu(z, "z");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(z.device());
+  TORCH_CHECK(z.is_contiguous() && out.is_cuda() && out.is_contiguous() && out.sizes() == z.sizes() &&
+              out.scalar_type() == z.scalar_type() && act_dtype(z) && out.device() == z.device(),
+              "kgc.relu_sq: shapes / dtypes");
+  kgc::launch_relu_sq(dt_code(z), out.data_ptr(), z.data_ptr(), z.numel(), stream());
+}
+
+void side_gate(Tensor out, Tensor pre, Tensor ids, Tensor table, int64_t col0) {
+  check_gpu(pre, "pre");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(pre.device());
+  TORCH_CHECK(pre.dim() == 2 && pre.is_contiguous() && act_dtype(pre) && out.is_cuda() &&
+              out.is_contiguous() && out.sizes() == pre.sizes() &&
+              out.scalar_type() == pre.scalar_type() && out.device() == pre.device(),
+              "kgc.side_gate: pre / out [T, n]");
+  const int64_t T = pre.size(0), n = pre.size(1);
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kLong && ids.numel() == T &&
+              ids.is_contiguous(), "kgc.side_gate: ids int64 [T]");
+  TORCH_CHECK(table.is_cuda() && table.dim() == 2 && table.stride(1) == 1 &&
+              table.scalar_type() == pre.scalar_type() && table.device() == pre.device() &&
+              col0 >= 0 && col0 + n <= table.size(1), "kgc.side_gate: table [vocab, >= col0 + n]");
+  kgc::launch_side_gate(dt_code(pre), out.data_ptr(), pre.data_ptr(), ids.data_ptr<int64_t>(),
+                        table.data_ptr(), table.stride(0), (int)table.size(0), (int)col0, (int)T,
+                        (int)n, stream());
+}
+
+void moe_route_sigmoid(Tensor w, Tensor ids, Tensor scores, Tensor correction, double scale) {
+  check_f32(w, "w");
+  check_f32(correction, "correction");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(w.device());
+  TORCH_CHECK(scores.is_cuda() && scores.scalar_type() == at::kFloat && scores.dim() == 2 &&
+              scores.stride(1) == 1 && scores.device() == w.device(), "kgc.moe_route_sigmoid: scores fp32 [T, >= E]");
+  const int64_t T = scores.size(0), E = correction.numel();
+  TORCH_CHECK(w.dim() == 2 && w.size(0) == T, "kgc.moe_route_sigmoid: w [T, k]");
+  const int64_t k = w.size(1);
+  TORCH_CHECK(E >= 1 && E <= scores.size(1) && E <= kgc::moe_route_sigmoid_max_experts() &&
+              k >= 1 && k <= E && k <= 64, "kgc.moe_route_sigmoid: experts / top");
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kInt && ids.is_contiguous() &&
+              ids.numel() == T * k && ids.device() == w.device(), "kgc.moe_route_sigmoid: ids int32 [T, k]");
+  kgc::launch_moe_route_sigmoid(w.data_ptr<float>(), ids.data_ptr<int>(), scores.data_ptr<float>(),
+                                scores.stride(0), correction.data_ptr<float>(), (int)T, (int)E,
+                                (int)k, (float)scale, stream());
+}
+
+void moe_finish(Tensor out, std::optional<Tensor> routed, std::optional<Tensor> dense,
+                std::optional<Tensor> topk_w, std::optional<Tensor> topk_ids,
+                std::optional<Tensor> shared, std::optional<Tensor> gate) {
+  check_gpu(out, "out");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(out.device());
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && act_dtype(out), "kgc.moe_finish: out [T, W]");
+  const int64_t T = out.size(0), W = out.size(1);
+  auto same = [&](const Tensor& t) {
+    return t.is_cuda() && t.is_contiguous() && t.scalar_type() == out.scalar_type() &&
+           t.device() == out.device();
+  };
+  const void *rp = nullptr, *dp = nullptr, *sp = nullptr;
+  const float *wp = nullptr, *gp = nullptr;
+  const int* ip = nullptr;
+  int64_t E = 0, k = 0, gs = 0;
+  if (routed.has_value()) {
+    TORCH_CHECK(same(*routed) && routed->sizes() == out.sizes(), "kgc.moe_finish: routed [T, W]");
+    rp = routed->data_ptr();
+  } else {
+    TORCH_CHECK(dense.has_value() && topk_w.has_value() && topk_ids.has_value(),
+                "kgc.moe_finish: routed, or dense + topk_w + topk_ids");
+    TORCH_CHECK(same(*dense) && dense->dim() == 3 && dense->size(1) == T && dense->size(2) == W,
+                "kgc.moe_finish: dense [E, T, W]");
+    E = dense->size(0);
+    check_f32(*topk_w, "topk_w");
+    TORCH_CHECK(topk_w->dim() == 2 && topk_w->size(0) == T, "kgc.moe_finish: topk_w [T, k]");
+    k = topk_w->size(1);
+    TORCH_CHECK(topk_ids->is_cuda() && topk_ids->scalar_type() == at::kInt &&
+                topk_ids->is_contiguous() && topk_ids->numel() == T * k, "kgc.moe_finish: topk_ids int32 [T, k]");
+    dp = dense->data_ptr();
+    wp = topk_w->data_ptr<float>();
+    ip = topk_ids->data_ptr<int>();
+  }
+  if (shared.has_value()) {
+    TORCH_CHECK(same(*shared) && shared->sizes() == out.sizes() && gate.has_value(),
+                "kgc.moe_finish: shared [T, W] with its gate");
+    TORCH_CHECK(gate->is_cuda() && gate->scalar_type() == at::kFloat && gate->dim() == 1 &&
+                gate->size(0) == T && gate->device() == out.device(), "kgc.moe_finish: gate fp32 [T]");
+    sp = shared->data_ptr();
+    gp = gate->data_ptr<float>();
+    gs = gate->stride(0);
+  }
+  kgc::launch_moe_finish(dt_code(out), out.data_ptr(), rp, dp, wp, ip, sp, gp, gs, (int)T, (int)E,
+                         (int)k, (int)W, stream());
+}
+
 }  // namespace
 
 TORCH_LIBRARY(kgc, m) {
+  m.def("residual_norm(Tensor(a!)? out, Tensor(b!) x, Tensor? add, Tensor? add_norm_w, Tensor? w, "
+        "float mult, float eps) -> ()");
+  m.def("token_shift(Tensor(a!) out, Tensor h, Tensor mu, Tensor(b!) state, Tensor? qsl, Tensor? seq_lens, "
+        "Tensor? ctx_lens, Tensor slots, int P, int D, int Tp) -> ()");
+  m.def("mingru_scan(Tensor(a!) out, Tensor zxg, Tensor bias, Tensor(b!) state, Tensor? qsl, "
+        "Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int width) -> ()");
+  m.def("latent_rope_store(Tensor(a!) q_out, Tensor proj, Tensor q_lat, Tensor positions, Tensor? table, "
+        "Tensor norm_w, float eps, Tensor(b!) cache, Tensor slots, int H, int d, int r, int rank) -> ()");
+  m.def("gate_mul(Tensor(a!) out, Tensor o, Tensor g) -> ()");
+  m.def("relu_sq(Tensor(a!) out, Tensor z) -> ()");
+  m.def("side_gate(Tensor(a!) out, Tensor pre, Tensor ids, Tensor table, int col0) -> ()");
+  m.def("moe_route_sigmoid(Tensor(a!) w, Tensor(b!) ids, Tensor scores, Tensor correction, float scale) -> ()");
+  m.def("moe_finish(Tensor(a!) out, Tensor? routed, Tensor? dense, Tensor? topk_w, Tensor? topk_ids, "
+        "Tensor? shared, Tensor? gate) -> ()");
   m.def("residual_group_norm(Tensor(a!) out, Tensor(b!) x, Tensor? y, Tensor w, int groups, float eps) -> ()");
   m.def("depth_mix_norm(Tensor(a!) out, Tensor(b!) x, Tensor(c!) hist, Tensor y, Tensor coef, Tensor w, "
         "int layer, int groups, float eps) -> ()");
@@ -1604,6 +1876,15 @@ TORCH_LIBRARY_IMPL(kgc, CUDA, m) {
   m.impl("rope_kv_store", &rope_kv_store);
   m.impl("window_attention", &window_attention);
   m.impl("mlstm_scan", &mlstm_scan);
+  m.impl("residual_norm", &residual_norm);
+  m.impl("token_shift", &token_shift);
+  m.impl("mingru_scan", &mingru_scan);
+  m.impl("latent_rope_store", &latent_rope_store);
+  m.impl("gate_mul", &gate_mul);
+  m.impl("relu_sq", &relu_sq);
+  m.impl("side_gate", &side_gate);
+  m.impl("moe_route_sigmoid", &moe_route_sigmoid);
+  m.impl("moe_finish", &moe_finish);
   m.impl("rms_norm", &rms_norm);
   m.impl("layer_norm", &layer_norm);
   m.impl("silu_mul", &silu_mul);

@@ -1,6 +1,7 @@
 // Windowed attention with kept first tokens over a plain-layout paged cache
 // (k [nb, G, bs, dk], v [nb, G, bs, dv]; dk != dv allowed, any sizes), for the hybrid
-// decoders.  Query i sees key j when j <= i and (i - j < window or j < keep_first);
+// decoders.  Rows are addressed through their strides (krs, vrs elements per cache row), so
+// the values may be columns of the key rows (one latent cache row per token).  Query i sees key j when j <= i and (i - j < window or j < keep_first);
 // window <= 0 means plain causal attention.
 //
 //   rope_kv_store     rotates q and k on the first `rot` dims of a head (pair i, i + rot/2;
@@ -70,8 +71,8 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const int* __restrict__ pbt, const int* __restrict__ ctx_lens, const int* __restrict__ dbt,
-    int bt_stride, int P, int Tp, int H, int G, int dk, int dv, int bs, int num_blocks,
-    float scale, int window, int keep_first, const float* __restrict__ gate, int kinds) {
+    int bt_stride, int P, int Tp, int H, int G, int dk, int dv, int krs, int vrs, int bs,
+    int num_blocks, float scale, int window, int keep_first, const float* __restrict__ gate, int kinds) {
   extern __shared__ float lds[];
   if (!(kinds & (blockIdx.x < Tp ? 1 : 2))) return;   // rows another kernel of the step owns
   float* qs = lds;                  // [dk]
@@ -119,7 +120,7 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
       int b = bt[j / bs];
       if (b < 0 || b >= num_blocks) b = 0;       // never index outside the pool
       ro = (b * G + g) * bs + (j % bs);
-      const T* kr = k_cache + (int64_t)ro * dk;
+      const T* kr = k_cache + (int64_t)ro * krs;
       float d = 0.f;
       for (int c = 0; c < dk; ++c) d += qs[c] * to_f(kr[c]);
       s = d * scale;
@@ -139,7 +140,7 @@ __global__ __launch_bounds__(64) void window_attention_kernel(
       const int c = lane + 64 * u;
       if (c < dv) {
         float a = acc[u] * alpha;
-        for (int jj = 0; jj < cnt; ++jj) a += pw[jj] * to_f(v_cache[(int64_t)voff[jj] * dv + c]);
+        for (int jj = 0; jj < cnt; ++jj) a += pw[jj] * to_f(v_cache[(int64_t)voff[jj] * vrs + c]);
         acc[u] = a;
       }
     }
@@ -226,8 +227,8 @@ template <typename T, int QH, int NWV>
 __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ ctx_lens, const int* __restrict__ dbt,
-    int bt_stride, int Tp, int H, int G, int dk, int dv, int bs, int num_blocks, float scale,
-    int window, int keep_first, const float* __restrict__ gate) {
+    int bt_stride, int Tp, int H, int G, int dk, int dv, int krs, int vrs, int bs, int num_blocks,
+    float scale, int window, int keep_first, const float* __restrict__ gate) {
   extern __shared__ float lds[];
   const int dd = blockIdx.x, g = blockIdx.y, qpg = H / G, hq0 = blockIdx.z * QH;
   const int nh = min(QH, qpg - hq0);
@@ -278,7 +279,7 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
       int b = bt[j / bs];
       if (b < 0 || b >= num_blocks) b = 0;
       ro = (b * G + g) * bs + (j % bs);
-      const T* kr = k_cache + (int64_t)ro * dk;
+      const T* kr = k_cache + (int64_t)ro * krs;
       constexpr int KB = 8;                       // 16-byte pieces of the key row in flight
       for (int c0 = 0; c0 < dk; c0 += 8 * KB) {
         Raw8<T> kraw[KB];
@@ -334,7 +335,7 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
 #pragma unroll
         for (int b = 0; b < VB; ++b) {
           const int jj = min(j0 + b * kg, cnt - 1);            // clamped: weight 0 below
-          raw[b] = load8raw(v_cache + (int64_t)ow[jj] * dv + 8 * ci);
+          raw[b] = load8raw(v_cache + (int64_t)ow[jj] * vrs + 8 * ci);
         }
 #pragma unroll
         for (int b = 0; b < VB; ++b) {
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
         }
         for (int jj = 0; jj < cnt; ++jj) {
           float v0, v1;
-          load2(v_cache + (int64_t)ow[jj] * dv + c0, v0, v1);
+          load2(v_cache + (int64_t)ow[jj] * vrs + c0, v0, v1);
 #pragma unroll
           for (int h = 0; h < QH; ++h) {
             const float p = pw[h * 64 + jj];
@@ -459,8 +460,8 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
     const int* __restrict__ pbt, int bt_stride, const int* __restrict__ work_seq,
-    const int* __restrict__ work_blk, int blk_rows, int H, int G, int dk, int dv, int bs,
-    int num_blocks, float scale, int window, int keep_first, const float* __restrict__ gate) {
+    const int* __restrict__ work_blk, int blk_rows, int H, int G, int dk, int dv, int krs,
+    int vrs, int bs, int num_blocks, float scale, int window, int keep_first, const float* __restrict__ gate) {
   typedef typename Vec8<T>::type V8;
   extern __shared__ float lds_f[];
   T* Ks = reinterpret_cast<T*>(lds_f);                 // [64][dk + 8]
@@ -521,7 +522,7 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
 #pragma unroll
     for (int kq = 0; kq < 4; ++kq) {
       const int ks = sr + 16 * kq, key = kb + ks;
-      const T* src = key < hi ? k_cache + page_row(key) * dk : nullptr;
+      const T* src = key < hi ? k_cache + page_row(key) * krs : nullptr;
       for (int c = sc; c < kchunks; c += 16) {
         u32x4 val = u32x4{0u, 0u, 0u, 0u};
         if (src != nullptr) val = *reinterpret_cast<const u32x4*>(src + 8 * c);
@@ -530,7 +531,7 @@ __global__ __launch_bounds__(256, KSM <= 4 ? 3 : 2) void window_prefill_mfma_ker
     }
     {
       const int ks = threadIdx.x & (PFW_BN - 1), key = kb + ks;   // a wave's lanes: consecutive keys
-      const T* src = key < hi ? v_cache + page_row(key) * dv : nullptr;
+      const T* src = key < hi ? v_cache + page_row(key) * vrs : nullptr;
       for (int c = threadIdx.x >> 6; c < vchunks; c += 4) {
         Pack8<T> val;
         val.u = u32x4{0u, 0u, 0u, 0u};
@@ -668,15 +669,15 @@ int window_attention_max_dv() { return 64 * MAX_DV_PER_LANE; }
 void launch_window_attention(int dtype, void* out, const void* q, const void* k_cache,
                              const void* v_cache, const int* qsl, const int* seq_lens,
                              const int* pbt, const int* ctx_lens, const int* dbt, int bt_stride,
-                             int P, int Tp, int T_, int H, int G, int dk, int dv, int bs,
-                             int num_blocks, float scale, int window, int keep_first,
+                             int P, int Tp, int T_, int H, int G, int dk, int dv, int krs, int vrs,
+                             int bs, int num_blocks, float scale, int window, int keep_first,
                              const float* gate, int kinds, hipStream_t s) {
   if (T_ <= 0 || !kinds) return;
   const size_t lds = (size_t)(dk + 128) * sizeof(float);
   KGC_DISPATCH_T(dtype, window_attention_kernel<T><<<dim3(T_, H), 64, lds, s>>>(
       (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache, qsl, seq_lens, pbt, ctx_lens,
-      dbt, bt_stride, P, Tp, H, G, dk, dv, bs, num_blocks, scale, window, keep_first, gate,
-      kinds));
+      dbt, bt_stride, P, Tp, H, G, dk, dv, krs, vrs, bs, num_blocks, scale, window, keep_first,
+      gate, kinds));
 }
 
 // decode rows on the 8-wave kernel: needs 16-byte key rows (dk % 8 == 0), even dv <= 512
@@ -693,7 +694,7 @@ static size_t decode_lds(int QH, int nwv, int dk, int dv) {
 template <typename T>
 static void decode_dispatch(T* out, const T* q, const T* kc, const T* vc, const int* ctx_lens,
                             const int* dbt, int bt_stride, int Tp, int D, int H, int G, int dk,
-                            int dv, int bs, int num_blocks, float scale, int window,
+                            int dv, int krs, int vrs, int bs, int num_blocks, float scale, int window,
                             int keep_first, const float* gate, hipStream_t s) {
   const int qpg = H / G;
   const int QH = qpg >= 8 ? 8 : qpg >= 3 ? 4 : qpg;      // heads per workgroup: 1, 2, 4, 8
@@ -703,8 +704,8 @@ static void decode_dispatch(T* out, const T* q, const T* kc, const T* vc, const 
   const bool small = (int64_t)grid.x * grid.y * grid.z >= 512;
 #define KGC_DEC(N, W)                                                                        \
   window_decode_kernel<T, N, W><<<grid, 64 * W, decode_lds(N, W, dk, dv), s>>>(              \
-      out, q, kc, vc, ctx_lens, dbt, bt_stride, Tp, H, G, dk, dv, bs, num_blocks, scale,     \
-      window, keep_first, gate)
+      out, q, kc, vc, ctx_lens, dbt, bt_stride, Tp, H, G, dk, dv, krs, vrs, bs, num_blocks,     \
+      scale, window, keep_first, gate)
 #define KGC_DEC2(N) \
   do {              \
     if (small) KGC_DEC(N, 4); else KGC_DEC(N, 8); \
@@ -724,13 +725,13 @@ size_t window_decode_lds(int dk, int dv, int qpg) {
 
 void launch_window_decode(int dtype, void* out, const void* q, const void* k_cache,
                           const void* v_cache, const int* ctx_lens, const int* dbt,
-                          int bt_stride, int Tp, int D, int H, int G, int dk, int dv, int bs,
-                          int num_blocks, float scale, int window, int keep_first,
+                          int bt_stride, int Tp, int D, int H, int G, int dk, int dv, int krs,
+                          int vrs, int bs, int num_blocks, float scale, int window, int keep_first,
                           const float* gate, hipStream_t s) {
   if (D <= 0) return;
   KGC_DISPATCH_T(dtype, decode_dispatch<T>((T*)out, (const T*)q, (const T*)k_cache,
                                            (const T*)v_cache, ctx_lens, dbt, bt_stride, Tp, D, H,
-                                           G, dk, dv, bs, num_blocks, scale, window, keep_first,
+                                           G, dk, dv, krs, vrs, bs, num_blocks, scale, window, keep_first,
                                            gate, s));
 }
 
@@ -749,14 +750,15 @@ template <typename T>
 static void prefill_dispatch(T* out, const T* q, const T* kc, const T* vc, const int* qsl,
                              const int* seq_lens, const int* pbt, int bt_stride,
                              const int* work_seq, const int* work_blk, int n_work, int blk_rows,
-                             int H, int G, int dk, int dv, int bs, int num_blocks, float scale,
-                             int window, int keep_first, const float* gate, hipStream_t s) {
+                             int H, int G, int dk, int dv, int krs, int vrs, int bs, int num_blocks,
+                             float scale, int window, int keep_first, const float* gate,
+                             hipStream_t s) {
   const dim3 grid(n_work * (blk_rows / PFW_BM), H);
   const size_t lds = window_prefill_mfma_lds(dk, dv);
 #define KGC_PF(K, D)                                                                          \
   window_prefill_mfma_kernel<T, K, D><<<grid, 256, lds, s>>>(                                 \
       out, q, kc, vc, qsl, seq_lens, pbt, bt_stride, work_seq, work_blk, blk_rows, H, G, dk,  \
-      dv, bs, num_blocks, scale, window, keep_first, gate)
+      dv, krs, vrs, bs, num_blocks, scale, window, keep_first, gate)
   if (dk <= 128 && dv <= 128) KGC_PF(4, 8);
   else KGC_PF(8, 16);
 #undef KGC_PF
@@ -766,18 +768,94 @@ void launch_window_prefill_mfma(int dtype, void* out, const void* q, const void*
                                 const void* v_cache, const int* qsl, const int* seq_lens,
                                 const int* pbt, int bt_stride, const int* work_seq,
                                 const int* work_blk, int n_work, int blk_rows, int H, int G,
-                                int dk, int dv, int bs, int num_blocks, float scale, int window,
+                                int dk, int dv, int krs, int vrs, int bs, int num_blocks, float scale, int window,
                                 int keep_first, const float* gate, hipStream_t s) {
   if (n_work <= 0) return;
   if (dtype == DT_BF16)
     prefill_dispatch<bf16>((bf16*)out, (const bf16*)q, (const bf16*)k_cache,
                            (const bf16*)v_cache, qsl, seq_lens, pbt, bt_stride, work_seq,
-                           work_blk, n_work, blk_rows, H, G, dk, dv, bs, num_blocks, scale,
-                           window, keep_first, gate, s);
+                           work_blk, n_work, blk_rows, H, G, dk, dv, krs, vrs, bs, num_blocks,
+                           scale, window, keep_first, gate, s);
   else
     prefill_dispatch<f16>((f16*)out, (const f16*)q, (const f16*)k_cache, (const f16*)v_cache,
                           qsl, seq_lens, pbt, bt_stride, work_seq, work_blk, n_work, blk_rows, H,
-                          G, dk, dv, bs, num_blocks, scale, window, keep_first, gate, s);
+                          G, dk, dv, krs, vrs, bs, num_blocks, scale, window, keep_first, gate, s);
+}
+
+// ---- latent attention: cache rows [normed latent | rotary key part] and query rows --------
+namespace {
+
+// One workgroup per token.  proj row: per head [d unrotated | r rotary] query columns, then
+// the latent pre-activation (rank) and the shared rotary key part (r).  q_lat [H, T, rank]
+// holds the unrotated query parts already multiplied into latent space.
+//   q_out [T, H, rank + r] = [q_lat | rotated query part]
+//   cache row (slot)       = [latent / rms(latent) * nw | rotated key part]
+// Rotary pairs are (2i, 2i + 1); table row = cos[r/2] | sin[r/2], fp32.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_rope_store_kernel(
+    T* __restrict__ q_out, const T* __restrict__ proj, int64_t proj_stride,
+    const T* __restrict__ q_lat, const int64_t* __restrict__ positions,
+    const float* __restrict__ table, int table_rows, const float* __restrict__ nw, float eps,
+    T* __restrict__ cache, const int64_t* __restrict__ slots, int64_t cache_rows, int T_, int H,
+    int d, int r, int rank) {
+  __shared__ float scratch[4];
+  const int64_t t = blockIdx.x;
+  const T* row = proj + t * proj_stride;
+  int64_t pos = positions[t];
+  if (pos < 0) pos = 0;
+  if (pos >= table_rows) pos = table_rows - 1;        // host checks max_pos; never read past
+  const float* cs = table != nullptr ? table + pos * r : nullptr;
+  const int half = r >> 1, dq = d + r, dk = rank + r;
+  for (int e = threadIdx.x; e < H * dk; e += 256) {
+    const int head = e / dk, i = e - head * dk;
+    float v;
+    if (i < rank) {
+      v = to_f(q_lat[((int64_t)head * T_ + t) * rank + i]);
+    } else {
+      const int j = i - rank, p = j >> 1;
+      const T* qr = row + head * dq + d;
+      float oa, ob;
+      neox_rot(to_f(qr[2 * p]), to_f(qr[2 * p + 1]), cs[p], cs[half + p], oa, ob);
+      v = (j & 1) ? ob : oa;
+    }
+    q_out[t * H * dk + e] = from_f<T>(v);
+  }
+  const int64_t slot = slots[t];
+  const T* kv = row + (int64_t)H * dq;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < rank; c += 256) {
+    const float v = to_f(kv[c]);
+    ss += v * v;
+  }
+  ss = block_sum<256>(ss, scratch);
+  if (slot < 0 || slot >= cache_rows) return;
+  const float rn = 1.f / sqrtf(ss / (float)rank + eps);
+  T* crow = cache + slot * dk;
+  for (int c = threadIdx.x; c < dk; c += 256) {
+    float v;
+    if (c < rank) {
+      v = to_f(kv[c]) * rn * nw[c];
+    } else {
+      const int j = c - rank, p = j >> 1;
+      float oa, ob;
+      neox_rot(to_f(kv[rank + 2 * p]), to_f(kv[rank + 2 * p + 1]), cs[p], cs[half + p], oa, ob);
+      v = (j & 1) ? ob : oa;
+    }
+    crow[c] = from_f<T>(v);
+  }
+}
+
+}  // namespace
+
+void launch_latent_rope_store(int dtype, void* q_out, const void* proj, int64_t proj_stride,
+                              const void* q_lat, const int64_t* positions, const float* table,
+                              int table_rows, const float* nw, float eps, void* cache,
+                              const int64_t* slots, int64_t cache_rows, int T_, int H, int d,
+                              int r, int rank, hipStream_t s) {
+  if (T_ <= 0) return;
+  KGC_DISPATCH_T(dtype, latent_rope_store_kernel<T><<<T_, 256, 0, s>>>(
+      (T*)q_out, (const T*)proj, proj_stride, (const T*)q_lat, positions, table, table_rows, nw,
+      eps, (T*)cache, slots, cache_rows, T_, H, d, r, rank));
 }
 
 }  // namespace kgc

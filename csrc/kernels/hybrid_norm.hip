@@ -6,6 +6,8 @@
 //   head_norm_gate       per-head RMS norm of a recurrence output, weight, sigmoid gate
 //   xielu                the xIELU activation
 //   gate_proj            a few fp32 gate outputs per row: act(h . w^T + b)
+//   residual_norm        x += mult * (add, or RMS-normed add * weight); h = RMSNorm(x) * w
+//   gate_mul, relu_sq, side_gate   element-wise epilogues between GEMMs
 // All arithmetic is fp32; T is the activation dtype of h / y (bf16, f16 or fp32).
 // One workgroup per row; a row is walked twice (sum of squares, then scale), the second
 // walk re-reading what the same thread wrote in the first.
@@ -264,6 +266,122 @@ void launch_gate_proj(int dtype, float* out, const void* h, const void* w, const
   const dim3 grid(rows, (N + NT / 64 - 1) / (NT / 64));
   KGC_DISPATCH_T(dtype, gate_proj_kernel<T><<<grid, NT, lds, s>>>(
       out, (const T*)h, (const T*)w, bias, W, N, kind_a, kind_b, split, cap));
+}
+
+// ---- scaled residual + plain RMS norm, head gate, squared ReLU, side-input gate ----------
+namespace {
+
+// x += mult * a, a = add or add / rms(add) * anw; then out = x / rms(x) * w (w null: x;
+// out null: none).  out may be x itself (O = float).  A thread touches the same columns
+// in every pass, so it re-reads only what it wrote.
+template <typename T, typename O>
+__global__ __launch_bounds__(NT) void residual_norm_kernel(
+    O* out, float* x, const T* __restrict__ add, const float* __restrict__ anw,
+    const float* __restrict__ w, float mult, int W, float eps) {
+  __shared__ float scratch[NT / 64];
+  const int64_t row = blockIdx.x;
+  float* xr = x + row * W;
+  if (add != nullptr) {
+    const T* ar = add + row * W;
+    if (anw != nullptr) {
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < W; c += NT) {
+        const float v = to_f(ar[c]);
+        ss += v * v;
+      }
+      ss = block_sum<NT>(ss, scratch);
+      const float ra = 1.f / sqrtf(ss / (float)W + eps);
+      for (int c = threadIdx.x; c < W; c += NT) xr[c] += mult * (to_f(ar[c]) * ra * anw[c]);
+    } else {
+      for (int c = threadIdx.x; c < W; c += NT) xr[c] += mult * to_f(ar[c]);
+    }
+  }
+  if (out == nullptr) return;
+  O* o = out + row * W;
+  if (w == nullptr) {
+    for (int c = threadIdx.x; c < W; c += NT) o[c] = from_f<O>(xr[c]);
+    return;
+  }
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += NT) ss += xr[c] * xr[c];
+  ss = block_sum<NT>(ss, scratch);
+  const float r = 1.f / sqrtf(ss / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += NT) o[c] = from_f<O>(xr[c] * r * w[c]);
+}
+
+// out [T, H * dv] = o[t, h, :] (strides st, sh) * sigmoid(g[t, h * dv + :]) (row stride sg)
+template <typename T>
+__global__ __launch_bounds__(NT) void gate_mul_kernel(
+    T* __restrict__ out, const T* __restrict__ o, int64_t st, int64_t sh,
+    const T* __restrict__ g, int64_t sg, int H, int dv) {
+  const int64_t t = blockIdx.x;
+  const int n = H * dv;
+  for (int e = threadIdx.x; e < n; e += NT) {
+    const int h = e / dv, c = e - h * dv;
+    const float gate = 1.f / (1.f + expf(-to_f(g[t * sg + e])));
+    out[t * n + e] = from_f<T>(to_f(o[t * st + h * sh + c]) * gate);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(NT) void relu_sq_kernel(T* __restrict__ out, const T* __restrict__ z,
+                                                     int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * NT + threadIdx.x; i < n; i += (int64_t)gridDim.x * NT) {
+    const float v = fmaxf(to_f(z[i]), 0.f);
+    out[i] = from_f<T>(v * v);
+  }
+}
+
+// out [T, n] = gelu_tanh(pre [T, n]) * table[ids[t], col0 + :] (table row stride ts)
+template <typename T>
+__global__ __launch_bounds__(NT) void side_gate_kernel(
+    T* __restrict__ out, const T* __restrict__ pre, const int64_t* __restrict__ ids,
+    const T* __restrict__ table, int64_t ts, int vocab, int col0, int n) {
+  const int64_t t = blockIdx.x;
+  int64_t id = ids[t];
+  if (id < 0 || id >= vocab) id = 0;                  // never read outside the table
+  const T* e = table + id * ts + col0;
+  for (int c = threadIdx.x; c < n; c += NT) {
+    const float z = to_f(pre[t * n + c]);
+    const float gl = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    out[t * n + c] = from_f<T>(gl * to_f(e[c]));
+  }
+}
+
+}  // namespace
+
+void launch_residual_norm(int dtype, int out_dtype, void* out, float* x, const void* add,
+                          const float* anw, const float* w, float mult, int rows, int W,
+                          float eps, hipStream_t s) {
+  if (rows <= 0) return;
+  if (out == nullptr || out_dtype == DT_F32) {
+    KGC_DISPATCH_T(dtype, residual_norm_kernel<T, float><<<rows, NT, 0, s>>>(
+        (float*)out, x, (const T*)add, anw, w, mult, W, eps));
+  } else {
+    KGC_DISPATCH_T(dtype, residual_norm_kernel<T, T><<<rows, NT, 0, s>>>(
+        (T*)out, x, (const T*)add, anw, w, mult, W, eps));
+  }
+}
+
+void launch_gate_mul(int dtype, void* out, const void* o, int64_t st, int64_t sh, const void* g,
+                     int64_t sg, int rows, int H, int dv, hipStream_t s) {
+  if (rows <= 0) return;
+  KGC_DISPATCH_T(dtype, gate_mul_kernel<T><<<rows, NT, 0, s>>>((T*)out, (const T*)o, st, sh,
+                                                              (const T*)g, sg, H, dv));
+}
+
+void launch_relu_sq(int dtype, void* out, const void* z, int64_t n, hipStream_t s) {
+  if (n <= 0) return;
+  const int grid = (int)std::min<int64_t>((n + NT - 1) / NT, 256 * 32);
+  KGC_DISPATCH_T(dtype, relu_sq_kernel<T><<<grid, NT, 0, s>>>((T*)out, (const T*)z, n));
+}
+
+void launch_side_gate(int dtype, void* out, const void* pre, const int64_t* ids,
+                      const void* table, int64_t ts, int vocab, int col0, int rows, int n,
+                      hipStream_t s) {
+  if (rows <= 0) return;
+  KGC_DISPATCH_T(dtype, side_gate_kernel<T><<<rows, NT, 0, s>>>(
+      (T*)out, (const T*)pre, ids, (const T*)table, ts, vocab, col0, n));
 }
 
 }  // namespace kgc

@@ -271,8 +271,8 @@ int window_attention_max_dv();
 void launch_window_attention(int dtype, void* out, const void* q, const void* k_cache,
                              const void* v_cache, const int* qsl, const int* seq_lens,
                              const int* pbt, const int* ctx_lens, const int* dbt, int bt_stride,
-                             int P, int Tp, int T, int H, int G, int dk, int dv, int bs,
-                             int num_blocks, float scale, int window, int keep_first,
+                             int P, int Tp, int T, int H, int G, int dk, int dv, int krs, int vrs,
+                             int bs, int num_blocks, float scale, int window, int keep_first,
                              const float* gate, int kinds, hipStream_t s);
 // `kinds` above: bit 0 = run the prefill rows, bit 1 = run the decode rows (the simple kernel
 // covers whatever the two kernels below do not take)
@@ -280,20 +280,52 @@ bool window_decode_ok(int dk, int dv, int qpg);
 size_t window_decode_lds(int dk, int dv, int qpg);
 void launch_window_decode(int dtype, void* out, const void* q, const void* k_cache,
                           const void* v_cache, const int* ctx_lens, const int* dbt,
-                          int bt_stride, int Tp, int D, int H, int G, int dk, int dv, int bs,
-                          int num_blocks, float scale, int window, int keep_first,
+                          int bt_stride, int Tp, int D, int H, int G, int dk, int dv, int krs,
+                          int vrs, int bs, int num_blocks, float scale, int window, int keep_first,
                           const float* gate, hipStream_t s);
 bool window_prefill_mfma_ok(int dtype, int dk, int dv);
 void launch_window_prefill_mfma(int dtype, void* out, const void* q, const void* k_cache,
                                 const void* v_cache, const int* qsl, const int* seq_lens,
                                 const int* pbt, int bt_stride, const int* work_seq,
                                 const int* work_blk, int n_work, int blk_rows, int H, int G,
-                                int dk, int dv, int bs, int num_blocks, float scale, int window,
+                                int dk, int dv, int krs, int vrs, int bs, int num_blocks, float scale, int window,
                                 int keep_first, const float* gate, hipStream_t s);
 int mlstm_scan_max_dim();
 void launch_mlstm_scan(int dtype, float* out, const void* qkvg, int64_t stride,
                        const float* gates, float* S, float* nst, float* mst, const int* qsl,
                        const int* seq_lens, const int* ctx_lens, const int* slots, int P, int D,
                        int Tp, int H, int d, int dv, int num_slots, hipStream_t s);
+
+// ---- scaled residual stream, token shift, minGRU, latent attention rows, sigmoid routing --
+// `dtype`: activation type of add / proj / zxg ...; `out_dtype`: DT_F32 or the same
+void launch_residual_norm(int dtype, int out_dtype, void* out, float* x, const void* add,
+                          const float* anw, const float* w, float mult, int rows, int W,
+                          float eps, hipStream_t s);
+void launch_gate_mul(int dtype, void* out, const void* o, int64_t st, int64_t sh, const void* g,
+                     int64_t sg, int rows, int H, int dv, hipStream_t s);
+void launch_relu_sq(int dtype, void* out, const void* z, int64_t n, hipStream_t s);
+void launch_side_gate(int dtype, void* out, const void* pre, const int64_t* ids,
+                      const void* table, int64_t ts, int vocab, int col0, int rows, int n,
+                      hipStream_t s);
+void launch_token_shift(int out_dtype, void* out, const float* h, const float* mu, float* state,
+                        const int* qsl, const int* seq_lens, const int* ctx_lens,
+                        const int* slots, int P, int Tp, int T, int W, int num_slots,
+                        hipStream_t s);
+void launch_mingru_scan(int dtype, void* out, const void* zxg, int64_t stride, const float* bias,
+                        float* state, const int* qsl, const int* seq_lens, const int* ctx_lens,
+                        const int* slots, int P, int D, int Tp, int width, int num_slots,
+                        hipStream_t s);
+void launch_latent_rope_store(int dtype, void* q_out, const void* proj, int64_t proj_stride,
+                              const void* q_lat, const int64_t* positions, const float* table,
+                              int table_rows, const float* nw, float eps, void* cache,
+                              const int64_t* slots, int64_t cache_rows, int T, int H, int d,
+                              int r, int rank, hipStream_t s);
+int moe_route_sigmoid_max_experts();
+void launch_moe_route_sigmoid(float* w, int* ids, const float* scores, int64_t stride,
+                              const float* corr, int ntok, int E, int k, float scale,
+                              hipStream_t s);
+void launch_moe_finish(int dtype, void* out, const void* routed, const void* dense,
+                       const float* w, const int* ids, const void* shared, const float* gate,
+                       int64_t gs, int ntok, int E, int k, int W, hipStream_t s);
 
 }  // namespace kgc

@@ -621,4 +621,118 @@ void launch_moe_combine(int dtype, void* out, const void* y, const float* topk_w
                                                   S, slice_stride);
 }
 
+// ---- sigmoid routing with a choice correction; combining dense expert outputs ------------
+namespace {
+
+// One wave per token.  scores fp32 [T, stride]: sigmoid router scores in the first E
+// columns.  k rounds of a wave-wide arg-max over score + correction (the lowest index
+// wins among equals); weights = the chosen scores / (their sum + 1e-20) * scale.
+constexpr int RS_MAX_PER_LANE = 16;          // E <= 1024
+
+__global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(
+    float* __restrict__ w, int* __restrict__ ids, const float* __restrict__ scores,
+    int64_t stride, const float* __restrict__ corr, int ntok, int E, int k, float scale) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= ntok) return;
+  const float* sr = scores + (int64_t)t * stride;
+  float sc[RS_MAX_PER_LANE], ch[RS_MAX_PER_LANE];
+#pragma unroll
+  for (int u = 0; u < RS_MAX_PER_LANE; ++u) {
+    const int e = lane + 64 * u;
+    sc[u] = e < E ? sr[e] : 0.f;
+    ch[u] = e < E ? sc[u] + corr[e] : -INFINITY;
+  }
+  float mine = 0.f, sum = 0.f;          // lane j keeps the j-th chosen score
+  int mine_id = 0;
+  for (int j = 0; j < k; ++j) {
+    float best = -INFINITY, bs = 0.f;
+    int bi = 0x7fffffff;
+#pragma unroll
+    for (int u = 0; u < RS_MAX_PER_LANE; ++u) {
+      if (ch[u] > best) {               // strict: the lowest index of a lane's equals
+        best = ch[u];
+        bi = lane + 64 * u;
+        bs = sc[u];
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ob = __shfl_xor(best, o, 64), os = __shfl_xor(bs, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ob > best || (ob == best && oi < bi)) {
+        best = ob;
+        bi = oi;
+        bs = os;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < RS_MAX_PER_LANE; ++u)
+      if (lane + 64 * u == bi) ch[u] = -INFINITY;
+    sum += bs;
+    if (j == lane) {                    // host checks k <= 64
+      mine = bs;
+      mine_id = bi < E ? bi : 0;
+    }
+  }
+  if (lane < k) {
+    w[(int64_t)t * k + lane] = mine / (sum + 1e-20f) * scale;
+    ids[(int64_t)t * k + lane] = mine_id;
+  }
+}
+
+// out[t] = routed[t] (already combined), or sum_j w[t, j] * dense[ids[t, j], t];
+// + gate[t * gs] * shared[t] when a shared expert is given.  fp32 sums.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_finish_kernel(
+    T* __restrict__ out, const T* __restrict__ routed, const T* __restrict__ dense,
+    const float* __restrict__ w, const int* __restrict__ ids, const T* __restrict__ shared,
+    const float* __restrict__ gate, int64_t gs, int ntok, int E, int k, int W) {
+  const int64_t t = blockIdx.x;
+  const float g = shared != nullptr ? gate[t * gs] : 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float acc = 0.f;
+    if (routed != nullptr) {
+      acc = to_f(routed[t * W + c]);
+    } else {
+      for (int j = 0; j < k; ++j) {
+        int e = ids[t * k + j];
+        if (e < 0 || e >= E) e = 0;
+        acc += w[t * k + j] * to_f(dense[((int64_t)e * ntok + t) * W + c]);
+      }
+    }
+    if (shared != nullptr) acc += g * to_f(shared[t * W + c]);
+    out[t * W + c] = from_f<T>(acc);
+  }
+}
+
+}  // namespace
+
+int moe_route_sigmoid_max_experts() { return 64 * RS_MAX_PER_LANE; }
+
+void launch_moe_route_sigmoid(float* w, int* ids, const float* scores, int64_t stride,
+                              const float* corr, int ntok, int E, int k, float scale,
+                              hipStream_t s) {
+  if (ntok <= 0) return;
+  moe_route_sigmoid_kernel<<<(ntok + 3) / 4, 256, 0, s>>>(w, ids, scores, stride, corr, ntok, E,
+                                                          k, scale);
+}
+
+void launch_moe_finish(int dtype, void* out, const void* routed, const void* dense,
+                       const float* w, const int* ids, const void* shared, const float* gate,
+                       int64_t gs, int ntok, int E, int k, int W, hipStream_t s) {
+  if (ntok <= 0) return;
+  if (dtype == DT_BF16)
+    moe_finish_kernel<bf16><<<ntok, 256, 0, s>>>((bf16*)out, (const bf16*)routed,
+                                                 (const bf16*)dense, w, ids, (const bf16*)shared,
+                                                 gate, gs, ntok, E, k, W);
+  else if (dtype == DT_F16)
+    moe_finish_kernel<f16><<<ntok, 256, 0, s>>>((f16*)out, (const f16*)routed, (const f16*)dense,
+                                                w, ids, (const f16*)shared, gate, gs, ntok, E, k,
+                                                W);
+  else
+    moe_finish_kernel<float><<<ntok, 256, 0, s>>>((float*)out, (const float*)routed,
+                                                  (const float*)dense, w, ids,
+                                                  (const float*)shared, gate, gs, ntok, E, k, W);
+}
+
 }  // namespace kgc

@@ -233,4 +233,164 @@ void launch_mlstm_scan(int dtype, float* out, const void* qkvg, int64_t stride,
                          ctx_lens, slots, P, D, Tp, H, d, dv, num_slots, s);
 }
 
+// ---- token shift and minGRU over per-sequence state vectors -----------------------------
+namespace {
+
+// The step sequence that holds row t: prefill chunk i (rows [qsl[i], qsl[i + 1])) or decode
+// row t - Tp.  first / last: the chunk's first and last row; pos0: position of the first.
+struct SeqOfRow { int idx, first, last, pos0; };
+
+__device__ __forceinline__ SeqOfRow seq_of_row(int t, const int* qsl, const int* seq_lens,
+                                               const int* ctx_lens, int P, int Tp) {
+  SeqOfRow r;
+  if (t < Tp) {
+    int lo = 0, hi = P - 1;
+    while (lo < hi) {
+      const int mid = (lo + hi + 1) >> 1;
+      if (qsl[mid] <= t) lo = mid; else hi = mid - 1;
+    }
+    r.idx = lo;
+    r.first = qsl[lo];
+    r.last = qsl[lo + 1] - 1;
+    r.pos0 = seq_lens[lo] - (qsl[lo + 1] - qsl[lo]);
+  } else {
+    r.idx = P + (t - Tp);
+    r.first = r.last = t;
+    r.pos0 = ctx_lens[t - Tp] - 1;
+  }
+  return r;
+}
+
+// One workgroup per row: out = h + (prev - h) * mu.  The workgroup of a chunk's first row
+// is the only one that touches the sequence's state: it reads the previous step's last row
+// from it and then stores this chunk's last row, so no other workgroup races with it.
+template <typename O>
+__global__ __launch_bounds__(NT) void token_shift_kernel(
+    O* __restrict__ out, const float* __restrict__ h, const float* __restrict__ mu,
+    float* __restrict__ state, const int* __restrict__ qsl, const int* __restrict__ seq_lens,
+    const int* __restrict__ ctx_lens, const int* __restrict__ slots, int P, int Tp, int W,
+    int num_slots) {
+  const int t = blockIdx.x;
+  const SeqOfRow sq = seq_of_row(t, qsl, seq_lens, ctx_lens, P, Tp);
+  const int slot = slots[sq.idx];
+  O* o = out + (int64_t)t * W;
+  if (slot < 0 || slot >= num_slots) {                 // a padding row
+    for (int c = threadIdx.x; c < W; c += NT) o[c] = from_f<O>(0.f);
+    return;
+  }
+  const float* hr = h + (int64_t)t * W;
+  if (t != sq.first) {
+    const float* pr = hr - W;
+    for (int c = threadIdx.x; c < W; c += NT) {
+      const float cur = hr[c];
+      o[c] = from_f<O>(cur + (pr[c] - cur) * mu[c]);
+    }
+    return;
+  }
+  float* st = state + (int64_t)slot * W;
+  const float* lr = h + (int64_t)sq.last * W;
+  const bool fresh = sq.pos0 <= 0;
+  for (int c = threadIdx.x; c < W; c += NT) {
+    const float cur = hr[c];
+    const float prev = fresh ? 0.f : st[c];
+    o[c] = from_f<O>(cur + (prev - cur) * mu[c]);
+    st[c] = lr[c];
+  }
+}
+
+__device__ __forceinline__ float sigmoidf_(float v) { return 1.f / (1.f + expf(-v)); }
+
+// grid (step sequences, ceil(width / 64)), one wave: lane = channel, tokens in order, the
+// loads of MG_UNROLL tokens in flight ahead of the dependent S chain.
+constexpr int MG_UNROLL = 8;
+
+template <typename T>
+__global__ __launch_bounds__(64) void mingru_scan_kernel(
+    T* __restrict__ out, const T* __restrict__ zxg, int64_t stride,
+    const float* __restrict__ bias, float* __restrict__ state, const int* __restrict__ qsl,
+    const int* __restrict__ seq_lens, const int* __restrict__ ctx_lens,
+    const int* __restrict__ slots, int P, int Tp, int width, int num_slots) {
+  const int s = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+  if (c >= width) return;
+  int start, len, pos0;
+  if (s < P) {
+    start = qsl[s];
+    len = qsl[s + 1] - start;
+    pos0 = seq_lens[s] - len;
+  } else {
+    start = Tp + (s - P);
+    len = 1;
+    pos0 = ctx_lens[s - P] - 1;
+  }
+  const int slot = slots[s];
+  if (slot < 0 || slot >= num_slots) {                 // a padding row
+    for (int t = start; t < start + len; ++t) out[(int64_t)t * width + c] = from_f<T>(0.f);
+    return;
+  }
+  float* st = state + (int64_t)slot * width + c;
+  float S = pos0 <= 0 ? 0.f : *st;
+  const float bz = bias[c], bx = bias[width + c];
+  for (int t0 = 0; t0 < len; t0 += MG_UNROLL) {
+    float zv[MG_UNROLL], uv[MG_UNROLL], gv[MG_UNROLL];
+#pragma unroll
+    for (int u = 0; u < MG_UNROLL; ++u) {
+      const int t = start + min(t0 + u, len - 1);
+      const T* row = zxg + (int64_t)t * stride;
+      zv[u] = to_f(row[c]);
+      uv[u] = to_f(row[width + c]);
+      gv[u] = to_f(row[2 * width + c]);
+    }
+#pragma unroll
+    for (int u = 0; u < MG_UNROLL; ++u) {
+      if (t0 + u < len) {
+        const float z = sigmoidf_(zv[u] + bz);
+        const float x = uv[u] + bx;
+        const float cand = x >= 0.f ? x + 0.5f : sigmoidf_(x);
+        S = (1.f - z) * S + z * cand;
+        const float g = gv[u];
+        out[(int64_t)(start + t0 + u) * width + c] = from_f<T>(S * (g * sigmoidf_(g)));
+      }
+    }
+  }
+  *st = S;
+}
+
+}  // namespace
+
+void launch_token_shift(int out_dtype, void* out, const float* h, const float* mu, float* state,
+                        const int* qsl, const int* seq_lens, const int* ctx_lens,
+                        const int* slots, int P, int Tp, int T_, int W, int num_slots,
+                        hipStream_t s) {
+  if (T_ <= 0) return;
+  if (out_dtype == DT_BF16)
+    token_shift_kernel<bf16><<<T_, NT, 0, s>>>((bf16*)out, h, mu, state, qsl, seq_lens, ctx_lens,
+                                               slots, P, Tp, W, num_slots);
+  else if (out_dtype == DT_F16)
+    token_shift_kernel<f16><<<T_, NT, 0, s>>>((f16*)out, h, mu, state, qsl, seq_lens, ctx_lens,
+                                              slots, P, Tp, W, num_slots);
+  else
+    token_shift_kernel<float><<<T_, NT, 0, s>>>((float*)out, h, mu, state, qsl, seq_lens,
+                                                ctx_lens, slots, P, Tp, W, num_slots);
+}
+
+void launch_mingru_scan(int dtype, void* out, const void* zxg, int64_t stride, const float* bias,
+                        float* state, const int* qsl, const int* seq_lens, const int* ctx_lens,
+                        const int* slots, int P, int D, int Tp, int width, int num_slots,
+                        hipStream_t s) {
+  if (P + D <= 0) return;
+  const dim3 grid(P + D, (width + 63) / 64);
+  if (dtype == DT_BF16)
+    mingru_scan_kernel<bf16><<<grid, 64, 0, s>>>((bf16*)out, (const bf16*)zxg, stride, bias, state,
+                                                 qsl, seq_lens, ctx_lens, slots, P, Tp, width,
+                                                 num_slots);
+  else if (dtype == DT_F16)
+    mingru_scan_kernel<f16><<<grid, 64, 0, s>>>((f16*)out, (const f16*)zxg, stride, bias, state,
+                                                qsl, seq_lens, ctx_lens, slots, P, Tp, width,
+                                                num_slots);
+  else
+    mingru_scan_kernel<float><<<grid, 64, 0, s>>>((float*)out, (const float*)zxg, stride, bias,
+                                                  state, qsl, seq_lens, ctx_lens, slots, P, Tp,
+                                                  width, num_slots);
+}
+
 }  // namespace kgc

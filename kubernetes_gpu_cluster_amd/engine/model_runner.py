@@ -245,23 +245,24 @@ class ModelRunner:
 
     def state_bytes(self) -> int:
         """Bytes of the recurrent layers' per-sequence state (one slot per sequence)."""
-        return sum(4 * self.max_num_seqs * (h * d * dv + h * d + h)
-                   for h, d, dv in self.state_layout)
+        return sum(4 * self.max_num_seqs * math.prod(shape)
+                   for shapes in self.state_layout for shape in shapes)
 
     def _init_states(self) -> None:
-        """Per recurrent layer (S [slots, H, d, dv], n [slots, H, d], m [slots, H]) in fp32.
-        Zero-filled once; a sequence's first token restarts its slot from zero by itself."""
+        """Per stateful layer run a tuple of fp32 tensors [slots, *shape], the shapes given
+        by the model's ``state_layout`` (mLSTM: S [H, d, dv], n [H, d], m [H]; minGRU and
+        token shift: one vector).  Zero-filled once; a sequence's first token restarts its
+        slot from zero by itself."""
         n = self.max_num_seqs
-        self.states = [(torch.zeros(n, h, d, dv, dtype=torch.float32, device=self.device),
-                        torch.zeros(n, h, d, dtype=torch.float32, device=self.device),
-                        torch.zeros(n, h, dtype=torch.float32, device=self.device))
-                       for h, d, dv in self.state_layout]
+        self.states = [tuple(torch.zeros(n, *shape, dtype=torch.float32, device=self.device)
+                             for shape in shapes) for shapes in self.state_layout]
 
     def init_kv_cache(self, num_blocks: int) -> None:
         m = self.model
         self._init_states()
         if self.cache_layout is not None:
             # plain row-major pages per attention layer: k [nb, G, bs, dk], v [nb, G, bs, dv]
+            # (dv = 0: the layer reads its values from columns of the key rows)
             self.kv = [(torch.zeros(num_blocks, g, self.bs, dk, dtype=self.kv_dtype,
                                     device=self.device),
                         torch.zeros(num_blocks, g, self.bs, dv, dtype=self.kv_dtype,

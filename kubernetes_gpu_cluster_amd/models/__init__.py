@@ -18,6 +18,7 @@ import torch
 
 from .configs import PRESETS, ModelConfig, resolve_model
 from .dilavik import DilavikForCausalLM
+from .konovik import KonovikForCausalLM
 from .llama import LlamaForCausalLM
 from .opt import OPTForCausalLM
 
@@ -27,6 +28,8 @@ def build_model(cfg: ModelConfig, dtype=torch.bfloat16, device=None):
         return OPTForCausalLM(cfg, dtype, device)
     if cfg.arch == "dilavik":
         return DilavikForCausalLM(cfg, dtype, device)
+    if cfg.arch == "konovik":
+        return KonovikForCausalLM(cfg, dtype, device)
     return LlamaForCausalLM(cfg, dtype, device)
 
 

@@ -128,3 +128,65 @@ class WindowedAttention(nn.Module):
         o = ops.window_attention(q, kc, vc, positions, ctx.attn, self.scale,
                                  w.size if w else 0, w.keep_first if w else 0, gate)
         return self.o_proj(o)
+
+
+class LatentAttention(nn.Module):
+    """Attention over a compressed cache: per token the cache row is one RMS-normed latent
+    c (``kv_rank`` wide) followed by one rotary key part (``rot_dims``) that all heads
+    share.  A head's key is [W_uk c | rotary part] and its value W_uv c, so
+        score = q_u . (W_uk c) + q_r . k_r = (W_uk^T q_u) . c + q_r . k_r
+    and   out = W_uv (sum_j p_j c_j):
+    the unrotated query part is multiplied into latent space (one batched GEMM per step),
+    all heads then attend the same rows as one key/value group -- keys are whole cache
+    rows, values their latent columns -- and a second batched GEMM lifts the result to the
+    heads' value size.  Prefill chunks and decode rows take the same path.  Sliding window,
+    softmax in fp32, ``scale`` as given; the concatenated heads are multiplied by
+    sigmoid(W_g h) before the output projection.
+
+    One merged projection yields q | latent + rotary key | gate.  The cache of a layer run
+    is chosen at call time (a looped layer has one per pass)."""
+
+    def __init__(self, hidden: int, spec, eps: float, dtype, device):
+        super().__init__()
+        from ..parallel.layers import ReplicatedLinear
+        self.spec, self.eps = spec, eps
+        H, d, r, dv, rank = spec.heads, spec.dim, spec.rot_dims, spec.vdim, spec.kv_rank
+        assert r % 2 == 0
+        self.n_q, self.n_kv, self.n_g = H * (d + r), rank + r, H * dv
+        self.proj = ReplicatedLinear(hidden, self.n_q + self.n_kv + self.n_g, dtype=dtype,
+                                     device=device)
+        self.o_proj = ReplicatedLinear(H * dv, hidden, dtype=dtype, device=device)
+        z = lambda *s: nn.Parameter(torch.zeros(*s, dtype=dtype, device=device),   # noqa: E731
+                                    requires_grad=False)
+        self.w_uk = z(H, d, rank)          # [head, unrotated dim, latent]: q_u -> latent space
+        self.w_uv = z(H, rank, dv)         # [head, latent, value dim]
+        self.norm_weight = nn.Parameter(torch.ones(rank, dtype=torch.float32, device=device),
+                                        requires_grad=False)
+        self.scale = (d + r) ** -0.5 if spec.scale is None else spec.scale
+        self.rope = None
+
+    def prepare(self, tables: dict, max_pos: int, device) -> None:
+        rs = self.spec.rotary
+        if rs is None:
+            return
+        key = (rs.dims, rs.base, rs.yarn)
+        if key not in tables:
+            tables[key] = ops.ref.rope_table_yarn(rs.dims, max_pos, rs.base, rs.yarn).to(device)
+        self.rope = tables[key]
+
+    def forward(self, h: torch.Tensor, positions: torch.Tensor, ctx: ForwardContext,
+                cache_idx: int):
+        sp = self.spec
+        H, d, r, dv, rank = sp.heads, sp.dim, sp.rot_dims, sp.vdim, sp.kv_rank
+        T = h.shape[0]
+        cache = ctx.kv_caches[cache_idx][0]                 # [nb, 1, bs, rank + r]
+        proj = self.proj(h)
+        qu = proj[:, : self.n_q].view(T, H, d + r)[:, :, :d].transpose(0, 1)   # [H, T, d]
+        q_lat = torch.bmm(qu, self.w_uk)                                       # [H, T, rank]
+        q = ops.latent_rope_store(proj, q_lat, positions, self.rope, self.norm_weight, self.eps,
+                                  cache, ctx.attn.slot_mapping, H, d, r, rank)
+        w = sp.window
+        o = ops.window_attention(q, cache, cache[..., :rank], positions, ctx.attn, self.scale,
+                                 w.size if w else 0, 0, None)                  # [T, H * rank]
+        o = torch.bmm(o.view(T, H, rank).transpose(0, 1), self.w_uv)           # [H, T, dv]
+        return self.o_proj(ops.gate_mul(o.transpose(0, 1), proj[:, self.n_q + self.n_kv:]))

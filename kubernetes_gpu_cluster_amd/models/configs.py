@@ -27,6 +27,36 @@ class WindowSpec:
 
 
 @dataclasses.dataclass(frozen=True)
+class RotarySpec:
+    """Rotary embedding of ``dims`` dimensions: pair i turns by p * base^(-2i/dims).
+    ``interleaved``: the pair is (2i, 2i + 1) instead of (i, i + dims/2).  ``yarn``
+    (factor, original length, fast turns, slow turns): YaRN frequency interpolation --
+    pairs that complete fewer than ``slow`` turns over the original length are slowed by
+    ``factor``, pairs above ``fast`` turns keep their frequency, a linear ramp between --
+    and cos / sin are scaled by 0.1 ln(factor) + 1."""
+    dims: int
+    base: float = 10000.0
+    interleaved: bool = False
+    yarn: Optional[tuple] = None
+
+
+@dataclasses.dataclass(frozen=True)
+class FeedForwardSpec:
+    """A layer's feed-forward.  kind "dense": gated, down(act(gate h) * up h).  kind "moe":
+    ``experts`` ungated experts down(act(up h)) of which a token uses ``top``: sigmoid
+    router scores, the choice made on score + a per-expert correction, the weights the
+    chosen scores over their sum times ``route_scale``; ``shared_ff`` > 0 adds an expert
+    every token uses, scaled by a per-token sigmoid gate."""
+    kind: str
+    ff: int
+    act: str = "silu"
+    experts: int = 0
+    top: int = 0
+    route_scale: float = 1.0
+    shared_ff: int = 0
+
+
+@dataclasses.dataclass(frozen=True)
 class MixerSpec:
     """One layer of a hybrid decoder: its token mixer and (optional) feed-forward.
 
@@ -34,7 +64,13 @@ class MixerSpec:
     size ``dim`` and value size ``vdim``, rotary on the first ``rot_dims`` dimensions,
     an optional window, an optional per-head sigmoid output gate).
     kind "mlstm": matrix-memory recurrence (one [dim, vdim] fp32 state per head and
-    sequence, exponential gating capped at ``gate_cap``)."""
+    sequence, exponential gating capped at ``gate_cap``).
+    kind "latent_attention": softmax attention whose keys and values are up-projections
+    of one ``kv_rank``-wide normed latent per token; a head's query / key has ``dim``
+    unrotated dimensions plus ``rot_dims`` rotated ones, the rotated key part shared by
+    all heads.  The paged cache holds the latent and the rotated key part only.
+    kind "mingru": an element-wise gated recurrence of ``width`` channels (one fp32 state
+    vector per sequence) with a SiLU output gate."""
     kind: str
     heads: int
     dim: int
@@ -48,6 +84,14 @@ class MixerSpec:
     gate_cap: float = 0.0
     ff: int = 0                  # 0: the layer has no feed-forward sublayer
     ff_kind: str = "dense"
+    kv_rank: int = 0             # latent_attention: width of the cached latent
+    width: int = 0               # mingru: recurrent channels
+    rotary: Optional[RotarySpec] = None     # latent_attention (rot_dims = rotary.dims)
+    mlp: Optional[FeedForwardSpec] = None   # feed-forwards other than the plain dense one
+
+    @property
+    def is_attention(self) -> bool:
+        return self.kind in ("attention", "latent_attention")
 
 
 @dataclasses.dataclass
@@ -85,6 +129,15 @@ class ModelConfig:
     layer_specs: Optional[tuple] = None
     norm_groups: int = 1
     embed_scale: float = 1.0
+    # arch "konovik": sublayer outputs join the stream times ``residual_mult``; layers
+    # [start, stop) of ``layer_loop`` = (start, stop, times) run ``times`` times in a row
+    # (own cache and state per pass); ``side_dim`` > 0: a per-layer, per-token embedding
+    # of that many columns gates a small projection after every layer; every mixer input
+    # is lerped towards the previous token's (``token_shift``, per-sequence state)
+    residual_mult: float = 1.0
+    layer_loop: Optional[tuple] = None
+    side_dim: int = 0
+    token_shift: bool = False
 
     @property
     def q_size(self) -> int:
@@ -102,19 +155,44 @@ class ModelConfig:
     def has_recurrent_state(self) -> bool:
         """A layer carries per-sequence state outside the paged KV cache: cached prefix
         blocks cannot stand in for computing the prefix."""
-        return any(sp.kind != "attention" for sp in (self.layer_specs or ()))
+        return self.token_shift or any(not sp.is_attention for sp in (self.layer_specs or ()))
+
+    def layer_runs(self) -> list:
+        """[(layer index, first layer of a repeated pass)] in execution order."""
+        n = len(self.layer_specs) if self.layer_specs else self.num_layers
+        if not self.layer_loop:
+            return [(i, False) for i in range(n)]
+        a, b, times = self.layer_loop
+        runs = [(i, False) for i in range(a)]
+        for k in range(times):
+            runs += [(i, k > 0 and i == a) for i in range(a, b)]
+        return runs + [(i, False) for i in range(b, n)]
 
     def num_params(self) -> int:
         h, i, L = self.hidden_size, self.intermediate_size, self.num_layers
         if self.layer_specs:
             n = 2 * self.vocab_size * h
             for sp in self.layer_specs:
-                if sp.kind == "attention":
+                if sp.kind == "latent_attention":
+                    n += h * (sp.heads * (sp.dim + sp.rot_dims) + sp.kv_rank + sp.rot_dims)
+                    n += sp.kv_rank * sp.heads * (sp.dim + sp.vdim) + 2 * h * sp.heads * sp.vdim
+                elif sp.kind == "mingru":
+                    n += 4 * h * sp.width
+                elif sp.kind == "attention":
                     n += h * (sp.heads * sp.dim + sp.kv_heads * (sp.dim + sp.vdim) + sp.heads)
                 else:
                     n += h * (2 * sp.heads * sp.dim + 2 * sp.heads * sp.vdim + 2 * sp.heads)
-                n += sp.heads * sp.vdim * h + 2 * h * sp.ff
-            return n
+                if sp.kind in ("attention", "mlstm"):
+                    n += sp.heads * sp.vdim * h
+                f = sp.mlp
+                if f is None:
+                    n += 2 * h * sp.ff
+                elif f.kind == "dense":
+                    n += 3 * h * f.ff
+                else:
+                    n += 2 * h * (f.experts * f.ff + f.shared_ff) + h * (f.experts + 1)
+                n += 2 * h * self.side_dim
+            return n + self.vocab_size * self.side_dim * len(self.layer_specs)
         attn = h * (self.q_size + 2 * self.kv_size) + self.q_size * h
         if self.act == "silu":
             mlp = 3 * h * i
@@ -127,8 +205,12 @@ class ModelConfig:
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
         if self.layer_specs:
-            return sum(sp.kv_heads * (sp.dim + sp.vdim) * dtype_bytes
-                       for sp in self.layer_specs if sp.kind == "attention")
+            n = {i: 0 for i in range(len(self.layer_specs))}
+            for i, _ in self.layer_runs():
+                n[i] += 1
+            return sum(n[i] * dtype_bytes * (sp.kv_rank + sp.rot_dims if sp.kind == "latent_attention"
+                                             else sp.kv_heads * (sp.dim + sp.vdim))
+                       for i, sp in enumerate(self.layer_specs) if sp.is_attention)
         return 2 * self.num_layers * self.num_kv_heads * self.head_dim * dtype_bytes
 
     def shrink(self, **kw) -> "ModelConfig":
@@ -288,10 +370,70 @@ def dilavik_config(d: dict, name: str) -> ModelConfig:
         bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)))
 
 
+def _feed_forward_spec(mlp: Optional[dict]) -> Optional[FeedForwardSpec]:
+    if not mlp:
+        return None
+    kind = mlp.get("kind", "dense")
+    if kind == "dense":
+        return FeedForwardSpec("dense", int(mlp["ff"]), act="silu")
+    if kind == "moe":
+        rt, sh = mlp["router"], mlp.get("shared")
+        return FeedForwardSpec("moe", int(mlp["expert"]["ff"]), act="relu2",
+                               experts=int(rt["experts"]), top=int(rt["top"]),
+                               route_scale=float(rt.get("scale", 1.0)),
+                               shared_ff=int(sh["ff"]) if sh else 0)
+    raise ValueError(f"unsupported feed-forward kind {kind!r}")
+
+
+def _konovik_spec(entry: dict) -> MixerSpec:
+    kind, m = entry["type"], entry["mixer"]
+    mlp = _feed_forward_spec(entry.get("mlp"))
+    ff = mlp.ff if mlp else 0
+    if kind == "latent_attention":
+        r = int(m.get("rot_dim", 0))
+        rot, mask = m.get("rot"), m.get("mask")
+        rs = None
+        if r:
+            sc = rot.get("scaling")
+            rs = RotarySpec(r, float(rot["base"]), interleaved=True,
+                            yarn=(float(sc["factor"]), float(sc["original"]), float(sc["fast"]),
+                                  float(sc["slow"])) if sc else None)
+        return MixerSpec("latent_attention", int(m["heads"]), int(m["dim"]), int(m["vdim"]),
+                         kv_heads=1, scale=float(m["scale"]), rot_dims=r,
+                         rot_base=rs.base if rs else 10000.0,
+                         window=WindowSpec(int(mask["size"])) if mask else None,
+                         ff=ff, kv_rank=int(m["kv_rank"]), rotary=rs, mlp=mlp)
+    if kind == "mingru":
+        return MixerSpec("mingru", 1, int(m["width"]), int(m["width"]), ff=ff,
+                         width=int(m["width"]), mlp=mlp)
+    raise ValueError(f"unknown mixer type {kind!r}")
+
+
+def konovik_config(d: dict, name: str) -> ModelConfig:
+    """A Konovik config.json (``architecture``, ``width``, ``vocab``, ``layers``, ``loop``,
+    ``norm``, ``residual_mult``, ``token_side``) -> ModelConfig."""
+    specs = tuple(_konovik_spec(e) for e in d["layers"])
+    att = next((sp for sp in specs if sp.is_attention), specs[0])
+    lp, side = d.get("loop"), d.get("token_side")
+    loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"])) if lp else None
+    if loop and not (0 <= loop[0] <= loop[1] <= len(specs) and loop[2] >= 1):
+        raise ValueError(f"bad layer loop {loop}")
+    return ModelConfig(
+        name, "konovik", len(specs), int(d["width"]), att.heads, 1, att.dim,
+        max((sp.ff for sp in specs), default=0), int(d["vocab"]),
+        max_position=int(d.get("max_position", 8192)), rope_theta=att.rot_base,
+        rms_eps=float(d["norm"]["eps"]), layer_specs=specs,
+        residual_mult=float(d.get("residual_mult", 1.0)), layer_loop=loop,
+        side_dim=int(side["dim"]) if side else 0, token_shift=True,
+        bos_token_id=int(d.get("bos_token_id", 0)), eos_token_id=int(d.get("eos_token_id", -1)))
+
+
 def _from_hf_config(d: dict, name: str) -> ModelConfig:
     """Map an HF config.json dict onto ModelConfig."""
     if d.get("architecture") == "Dilavik":
         return dilavik_config(d, name)
+    if d.get("architecture") == "Konovik":
+        return konovik_config(d, name)
     mt = d.get("model_type", "llama")
     if mt == "opt":
         h = d["hidden_size"]

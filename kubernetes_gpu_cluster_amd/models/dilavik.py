@@ -112,7 +112,7 @@ class DilavikForCausalLM(nn.Module):
                 if sp.kind == "attention"]
 
     def state_layout(self) -> list:
-        """(heads, dim, vdim) of every recurrent layer's per-sequence state."""
+        """Per recurrent layer, the per-slot shapes of its state tensors."""
         return [l.mix.state_shapes() for l in self.layers if isinstance(l.mix, MLSTMMixer)]
 
     def prepare(self, max_pos: int, max_tokens: int, device) -> None:

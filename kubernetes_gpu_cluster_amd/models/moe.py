@@ -262,3 +262,60 @@ class MoEBlock(nn.Module):
         w = topk_w.reshape(-1)[order]
         out.index_add_(0, tok, back.float() * w[:, None])
         return out.to(x.dtype)
+
+
+class SigmoidRoutedExperts(nn.Module):
+    """Mixture of ungated experts down(act(up h)) with sigmoid routing: scores
+    s = sigmoid(W_r h) in fp32; the ``top`` experts with the largest s + correction are
+    chosen; their weights are s / (sum of the chosen s + 1e-20) * route_scale.  An optional
+    shared expert of the same form runs for every token, scaled by sigmoid(w_sg . h).
+    Router and shared gate are one fp32 gate projection (rows: experts, then the gate).
+
+    Expert GEMMs: the grouped MFMA GEMM over expert-sorted rows where its tiles cover the
+    shapes (16-bit activations, ff % 128 == 0, hidden % 128 == 0); otherwise every expert
+    runs on every token as one batched GEMM pair and the chosen outputs are gathered -- no
+    host synchronisation either way, so decode graphs capture the block.  One GPU per
+    replica."""
+
+    def __init__(self, hidden: int, spec, dtype, device):
+        super().__init__()
+        assert spec.act == "relu2"
+        self.spec = spec
+        E, I = spec.experts, spec.ff
+        z = lambda *s: nn.Parameter(torch.zeros(*s, dtype=dtype, device=device),   # noqa: E731
+                                    requires_grad=False)
+        self.w_up = z(E, I, hidden)
+        self.w_down = z(E, hidden, I)
+        self.gates = z(E + (1 if spec.shared_ff else 0), hidden)
+        self.correction = nn.Parameter(torch.zeros(E, dtype=torch.float32, device=device),
+                                       requires_grad=False)
+        if spec.shared_ff:
+            self.shared_up = ReplicatedLinear(hidden, spec.shared_ff, dtype=dtype, device=device)
+            self.shared_down = ReplicatedLinear(spec.shared_ff, hidden, dtype=dtype, device=device)
+        else:
+            self.shared_up = self.shared_down = None
+        self.native = (torch.device(device).type == "cuda" and dtype != torch.float32 and
+                       ops.moe_supported(I, hidden) and ops.moe_supported(hidden, I))
+
+    def routed(self, x, topk_w, topk_ids):
+        """-> (combined [T, W] or None, per-expert outputs [E, T, W] or None)."""
+        if self.native and x.is_cuda:
+            return ops.grouped_experts(x, self.w_up, self.w_down, topk_w, topk_ids,
+                                       ops.relu_sq), None
+        T = x.shape[0]
+        xe = x.unsqueeze(0).expand(self.spec.experts, T, x.shape[1])
+        a = ops.relu_sq(torch.bmm(xe, self.w_up.transpose(1, 2)))
+        return None, torch.bmm(a, self.w_down.transpose(1, 2))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        sp = self.spec
+        scores = ops.gate_proj(x, self.gates, None, ops.GATE_SIGMOID)       # fp32 [T, E (+1)]
+        topk_w, topk_ids = ops.moe_route_sigmoid(scores, self.correction, sp.top, sp.route_scale)
+        routed, dense = self.routed(x, topk_w, topk_ids)
+        shared = gate = None
+        if self.shared_up is not None:
+            shared = self.shared_down(ops.relu_sq(self.shared_up(x)))
+            gate = scores[:, sp.experts]
+        if routed is not None and shared is None:
+            return routed
+        return ops.moe_finish(routed, dense, topk_w, topk_ids, shared, gate)

@@ -45,8 +45,9 @@ class MLSTMMixer(nn.Module):
                                         requires_grad=False)
 
     def state_shapes(self) -> tuple:
+        """Per-slot shapes of the state tensors S, n, m."""
         sp = self.spec
-        return (sp.heads, sp.dim, sp.vdim)
+        return ((sp.heads, sp.dim, sp.vdim), (sp.heads, sp.dim), (sp.heads,))
 
     def forward(self, h: torch.Tensor, positions: torch.Tensor, ctx: ForwardContext):
         sp = self.spec
@@ -57,3 +58,29 @@ class MLSTMMixer(nn.Module):
         o = ops.mlstm_scan(qkvg, gates, ctx.states[self.state_idx], ctx.attn, H, d, dv)
         g = qkvg[:, 2 * H * d + H * dv:]
         return self.o_proj(ops.head_norm_gate(o, g, self.norm_weight, H, self.eps, h.dtype))
+
+
+class MinGRUMixer(nn.Module):
+    """minGRU: an element-wise gated recurrence whose gates read only the current token.
+    z = sigmoid(W_z h + b_z); u = W_x h + b_x; candidate = u + 1/2 (u >= 0) or sigmoid(u);
+    S_t = (1 - z) S_(t-1) + z candidate; output W_o (S_t * silu(W_g h)).  One merged
+    projection yields z | u | g; biases, gates and the state (fp32 [slots, width]) stay in
+    fp32.  The state slot tensor of a layer run is chosen at call time."""
+
+    def __init__(self, hidden: int, spec, dtype, device):
+        super().__init__()
+        self.spec = spec
+        n = spec.width
+        self.zxg_proj = ReplicatedLinear(hidden, 3 * n, dtype=dtype, device=device)
+        self.o_proj = ReplicatedLinear(n, hidden, dtype=dtype, device=device)
+        self.zx_bias = nn.Parameter(torch.zeros(2 * n, dtype=torch.float32, device=device),
+                                    requires_grad=False)
+
+    def state_shapes(self) -> tuple:
+        return ((self.spec.width,),)
+
+    def forward(self, h: torch.Tensor, positions: torch.Tensor, ctx: ForwardContext,
+                state: torch.Tensor):
+        y = ops.mingru_scan(self.zxg_proj(h), self.zx_bias, state, ctx.attn, self.spec.width,
+                            h.dtype)
+        return self.o_proj(y)

@@ -780,3 +780,154 @@ def head_norm_gate(o: torch.Tensor, g: torch.Tensor, w: torch.Tensor, H: int, ep
     out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
     _k().head_norm_gate(out, o, g, w, H, eps)
     return out
+
+
+# ------------------------------------------------------------------ Konovik-style decoders
+# A residual stream scaled per sublayer, token shift and minGRU over per-sequence state
+# slots, latent attention (the paged cache holds one normed latent + one rotary key part
+# per token; values are the latent columns of the same rows), sigmoid routing with a
+# choice correction over squared-ReLU experts, and a per-token side input.
+def residual_norm(x: torch.Tensor, add: Optional[torch.Tensor], mult: float,
+                  w: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype],
+                  add_norm_w: Optional[torch.Tensor] = None,
+                  out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x fp32 [T, W], in place: x += mult * a (a = add, or RMS-normed add times
+    add_norm_w); returns RMSNorm(x) * w (w None: x) in out_dtype (None: no output).
+    ``out`` may be x itself (fp32): the stream is replaced by its normed value."""
+    if not _gpu(x):
+        r = ref.residual_norm(x, add, mult, w, eps, out_dtype, add_norm_w)
+        if out is not None and r is not None:
+            out.copy_(r)
+            return out
+        return r
+    if out is None and out_dtype is not None:
+        out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
+    _k().residual_norm(out, x, add, add_norm_w, w, float(mult), eps)
+    return out
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, meta,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """h fp32 [T, W] -> h + (previous row of the sequence - h) * mu in out_dtype; the row
+    before a chunk's first comes from state [slots, W] (zeros at position 0), which then
+    takes the chunk's last row."""
+    if not _gpu(h):
+        return ref.token_shift(h, mu, state, ref.step_sequences(meta), out_dtype)
+    out = torch.empty(h.shape, dtype=out_dtype, device=h.device)
+    _k().token_shift(out, h, mu, state, meta.query_start_loc, meta.prefill_seq_lens,
+                     meta.decode_ctx_lens, meta.state_slots, meta.num_prefills,
+                     meta.num_decodes, meta.num_prefill_tokens)
+    return out
+
+
+def mingru_scan(zxg: torch.Tensor, bias: torch.Tensor, state: torch.Tensor, meta, width: int,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """The minGRU recurrence over every step sequence's rows from / into state
+    [slots, width] fp32, times silu of the output-gate columns: zxg [T, 3 width] holds the
+    update-gate | candidate | output-gate pre-activations, bias fp32 [2 width]."""
+    if not _gpu(zxg):
+        return ref.mingru_scan(zxg, bias, state, ref.step_sequences(meta), width, out_dtype)
+    out = torch.empty(zxg.shape[0], width, dtype=out_dtype, device=zxg.device)
+    _k().mingru_scan(out, zxg, bias, state, meta.query_start_loc, meta.prefill_seq_lens,
+                     meta.decode_ctx_lens, meta.state_slots, meta.num_prefills,
+                     meta.num_decodes, meta.num_prefill_tokens, width)
+    return out
+
+
+def latent_rope_store(proj: torch.Tensor, q_lat: torch.Tensor, positions: torch.Tensor,
+                      table: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
+                      cache: torch.Tensor, slot_mapping: torch.Tensor, H: int, d: int, r: int,
+                      rank: int) -> torch.Tensor:
+    """Cache rows [normed latent | rotated key part] of the step's tokens, and their query
+    rows [T, H, rank + r] = [q_lat (H, T, rank) | rotated query part]; see
+    ``ref.latent_rope_store``."""
+    if not _gpu(proj):
+        return ref.latent_rope_store(proj, q_lat, positions, table, norm_w, eps, cache,
+                                     slot_mapping, H, d, r, rank)
+    q = torch.empty(proj.shape[0], H, rank + r, dtype=proj.dtype, device=proj.device)
+    _k().latent_rope_store(q, proj, q_lat, positions, table, norm_w, eps, cache, slot_mapping,
+                           H, d, r, rank)
+    return q
+
+
+def gate_mul(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """o [T, H, dv] (any token / head strides) * sigmoid(g [T, H dv], a column slice)."""
+    if not _gpu(o):
+        return ref.gate_mul(o, g)
+    T, H, dv = o.shape
+    out = torch.empty(T, H * dv, dtype=g.dtype, device=g.device)
+    _k().gate_mul(out, o, g)
+    return out
+
+
+def relu_sq(z: torch.Tensor) -> torch.Tensor:
+    if not _gpu(z):
+        return ref.relu_sq(z)
+    out = torch.empty_like(z)
+    _k().relu_sq(out, z.contiguous())
+    return out
+
+
+def moe_route_sigmoid(scores: torch.Tensor, correction: torch.Tensor, k: int, scale: float):
+    """(weights fp32 [T, k], expert ids int32 [T, k]) from sigmoid scores fp32 [T, >= E]."""
+    if not _gpu(scores):
+        return ref.moe_route_sigmoid(scores, correction, k, scale)
+    T = scores.shape[0]
+    w = torch.empty(T, k, dtype=torch.float32, device=scores.device)
+    ids = torch.empty(T, k, dtype=torch.int32, device=scores.device)
+    _k().moe_route_sigmoid(w, ids, scores, correction, float(scale))
+    return w, ids
+
+
+def grouped_experts(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
+                    topk_w: torch.Tensor, topk_ids: torch.Tensor, act) -> torch.Tensor:
+    """sum_j topk_w[t, j] * down_e(act(up_e x[t])), e = topk_ids[t, j], on the grouped MFMA
+    GEMM (``moe_align`` buckets, rows gathered for the up projection and scattered back
+    by the down projection, ``moe_combine``): ungated experts w_up [E, I, H], w_down
+    [E, H, I] with the activation ``act`` between.  No host synchronisation."""
+    k = _k()
+    T, H = x.shape
+    E, I = w_up.shape[0], w_up.shape[1]
+    topk = topk_ids.shape[1]
+    npairs = T * topk
+    bm = 64 if npairs <= 40 * E else 128
+    rows = (npairs + E * (bm - 1) + bm - 1) // bm * bm
+    dev = x.device
+    sorted_ids = torch.empty(rows, dtype=torch.int32, device=dev)
+    block_expert = torch.empty(rows // bm, dtype=torch.int32, device=dev)
+    meta = torch.empty(1, dtype=torch.int32, device=dev)
+    k.moe_align(sorted_ids, block_expert, meta, topk_ids.contiguous(), 0, E, bm)
+    inter = torch.zeros(rows, I, dtype=x.dtype, device=dev)
+    k.moe_gemm(inter, x.contiguous(), w_up, sorted_ids, block_expert, meta, npairs, topk, bm,
+               True, False)
+    a = act(inter)
+    S = moe_splitk(npairs, E, H, I, bm)
+    if S > 1:
+        y = torch.empty(S, npairs, H, dtype=torch.float32, device=dev)
+    else:
+        y = torch.empty(npairs, H, dtype=x.dtype, device=dev)
+    k.moe_gemm(y, a, w_down, sorted_ids, block_expert, meta, npairs, topk, bm, False, True, S)
+    out = torch.empty(T, H, dtype=x.dtype, device=dev)
+    k.moe_combine(out, y, topk_w.contiguous().float())
+    return out
+
+
+def moe_finish(routed, dense, topk_w, topk_ids, shared, gate) -> torch.Tensor:
+    """Weighted sum of the chosen experts (``routed`` [T, W], or gathered from ``dense``
+    [E, T, W]) + gate[t] * shared[t]."""
+    src = routed if routed is not None else dense
+    if not _gpu(src):
+        return ref.moe_finish(routed, dense, topk_w, topk_ids, shared, gate)
+    T, W = src.shape[-2], src.shape[-1]
+    out = torch.empty(T, W, dtype=src.dtype, device=src.device)
+    _k().moe_finish(out, routed, dense, topk_w, topk_ids, shared, gate)
+    return out
+
+
+def side_gate(pre: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int) -> torch.Tensor:
+    """gelu_tanh(pre [T, n]) * table[ids, col0:col0 + n]."""
+    if not _gpu(pre):
+        return ref.side_gate(pre, ids, table, col0)
+    out = torch.empty_like(pre)
+    _k().side_gate(out, pre.contiguous(), ids, table, col0)
+    return out

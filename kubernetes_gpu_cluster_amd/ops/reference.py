@@ -520,3 +520,186 @@ def head_norm_gate(o: torch.Tensor, g: torch.Tensor, w: torch.Tensor, H: int, ep
     oh = o.float().view(T, H, N // H)
     oh = oh * torch.rsqrt(oh.pow(2).mean(-1, keepdim=True) + eps)
     return (oh.view(T, N) * w.float() * torch.sigmoid(g.float())).to(out_dtype)
+
+
+# ---------------------------------------------------------------- Konovik-style decoders
+# (scaled residual + norm, token shift, minGRU scan, latent-attention cache rows with
+# YaRN / interleaved rotary, sigmoid routing with a choice correction, squared-ReLU
+# experts, per-token side input)
+def rope_table_yarn(rot_dims: int, max_pos: int, base: float, yarn=None) -> torch.Tensor:
+    """[max_pos, rot_dims] fp32: cos | sin of p * f_i, i < rot_dims/2.  ``yarn`` =
+    (factor, original, fast, slow): f_i = base^(-2i/dims) is slowed by ``factor`` for the
+    pairs past the ramp between the dimensions that make ``fast`` and ``slow`` turns over
+    ``original`` positions, and cos / sin are scaled by 0.1 ln(factor) + 1."""
+    i = torch.arange(rot_dims // 2, dtype=torch.float32)
+    f = torch.tensor(base, dtype=torch.float32) ** (-2.0 * i / rot_dims)
+    mag = 1.0
+    if yarn is not None:
+        factor, orig, fast, slow = yarn
+
+        def turn_dim(turns):
+            return rot_dims * math.log(orig / (2 * math.pi * turns)) / (2 * math.log(base))
+        lo = max(math.floor(turn_dim(fast)), 0)
+        hi = min(math.ceil(turn_dim(slow)), rot_dims - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    a = torch.arange(max_pos, dtype=torch.float32)[:, None] * f[None]
+    return torch.cat([a.cos() * mag, a.sin() * mag], dim=-1)
+
+
+def residual_norm(x: torch.Tensor, add: Optional[torch.Tensor], mult: float,
+                  w: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype],
+                  add_norm_w: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """x (fp32, in place) += mult * a, with a = add, or add / rms(add) * add_norm_w when
+    that weight is given; then returns x / rms(x) * w (w None: x itself) in out_dtype
+    (None: nothing).  rms(v) = sqrt(mean(v^2) + eps); fp32 math."""
+    if add is not None:
+        a = add.float()
+        if add_norm_w is not None:
+            a = a * torch.rsqrt(a.pow(2).mean(-1, keepdim=True) + eps) * add_norm_w.float()
+        x += mult * a
+    if out_dtype is None:
+        return None
+    if w is None:
+        return x.to(out_dtype)
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def step_sequences(meta) -> list:
+    """[(first row, rows, position of the first row, state slot)] of a step's sequences:
+    prefill chunks, then decode rows."""
+    P, D, tp = meta.num_prefills, meta.num_decodes, meta.num_prefill_tokens
+    seqs = []
+    slots = meta.state_slots[: P + D].tolist()
+    if P:
+        qsl, sl = meta.query_start_loc.tolist(), meta.prefill_seq_lens.tolist()
+        for i in range(P):
+            n = qsl[i + 1] - qsl[i]
+            seqs.append((qsl[i], n, sl[i] - n, slots[i]))
+    if D:
+        ctx = meta.decode_ctx_lens.tolist()
+        for i in range(D):
+            seqs.append((tp + i, 1, ctx[i] - 1, slots[P + i]))
+    return seqs
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, seqs: list,
+                out_dtype: torch.dtype) -> torch.Tensor:
+    """h fp32 [T, W] -> h + (prev - h) * mu, prev the sequence's previous row (before this
+    replacement): the row above, or for a chunk's first row state[slot] (zeros at position
+    0).  state[slot] then holds the chunk's last row.  Rows of slot < 0 give zeros."""
+    out = torch.zeros_like(h)
+    for a, n, p0, slot in seqs:
+        if slot < 0:
+            continue
+        first = torch.zeros_like(h[:1]) if p0 == 0 else state[slot][None]
+        prev = torch.cat([first, h[a:a + n - 1]], 0)
+        out[a:a + n] = h[a:a + n] + (prev - h[a:a + n]) * mu.float()
+        state[slot] = h[a + n - 1]
+    return out.to(out_dtype)
+
+
+def mingru_scan(zxg: torch.Tensor, bias: torch.Tensor, state: torch.Tensor, seqs: list,
+                width: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """zxg [T, 3 width]: pre-activations of the update gate | candidate | output gate;
+    bias fp32 [2 width] for the first two.  z = sigmoid(.), u -> u + 1/2 (u >= 0) or
+    sigmoid(u); S = (1 - z) S + z cand per sequence from state[slot] (zeros at position
+    0), written back; -> S * silu(g) [T, width].  fp32 math."""
+    T = zxg.shape[0]
+    zx = zxg[:, : 2 * width].float() + bias.float()
+    z = torch.sigmoid(zx[:, :width])
+    u = zx[:, width:]
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    g = zxg[:, 2 * width: 3 * width].float()
+    out = torch.zeros(T, width, dtype=torch.float32, device=zxg.device)
+    for a, n, p0, slot in seqs:
+        if slot < 0:
+            continue
+        S = torch.zeros(width) if p0 == 0 else state[slot].clone()
+        for t in range(a, a + n):
+            S = (1 - z[t]) * S + z[t] * cand[t]
+            out[t] = S
+        state[slot] = S
+    return (out * g * torch.sigmoid(g)).to(out_dtype)
+
+
+def _rot_pairs(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
+    """x [..., r] with pairs (2i, 2i+1); cs [..., r] = cos | sin."""
+    r = x.shape[-1]
+    c, s = cs[..., : r // 2], cs[..., r // 2:]
+    u, v = x[..., 0::2], x[..., 1::2]
+    return torch.stack([u * c - v * s, v * c + u * s], dim=-1).flatten(-2)
+
+
+def latent_rope_store(proj: torch.Tensor, q_lat: torch.Tensor, positions: torch.Tensor,
+                      table: Optional[torch.Tensor], norm_w: torch.Tensor, eps: float,
+                      cache: torch.Tensor, slot_mapping: torch.Tensor, H: int, d: int, r: int,
+                      rank: int) -> torch.Tensor:
+    """proj [T, H (d + r) + rank + r + ...]: per head the query's d unrotated and r rotary
+    columns, then the latent pre-activation (rank) and the shared rotary key part (r).
+    q_lat [H, T, rank]: the unrotated query parts already multiplied into latent space.
+    Writes the cache row [RMS-normed latent * norm_w | rotated key part] at slot_mapping
+    (< 0: none) into cache [nb, 1, bs, rank + r] and returns the query rows
+    [T, H, rank + r] = [q_lat | rotated query part] in proj's dtype.  Pairs are (2i, 2i+1)."""
+    T = proj.shape[0]
+    q = proj[:, : H * (d + r)].float().view(T, H, d + r)[..., d:]
+    dkv = proj[:, H * (d + r): H * (d + r) + rank + r].float()
+    c = dkv[:, :rank]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    kr = dkv[:, rank:]
+    if r:
+        cs = table[positions.long()]
+        q = _rot_pairs(q, cs[:, None, :])
+        kr = _rot_pairs(kr, cs)
+    bs = cache.shape[2]
+    ok = slot_mapping >= 0
+    sl = slot_mapping[ok].long()
+    cache[sl // bs, 0, sl % bs] = torch.cat([c, kr], -1)[ok].to(cache.dtype)
+    return torch.cat([q_lat.float().transpose(0, 1), q], -1).to(proj.dtype)
+
+
+def gate_mul(o: torch.Tensor, g: torch.Tensor) -> torch.Tensor:
+    """o [T, H, dv] (any strides) * sigmoid(g [T, H dv]) -> [T, H dv] in g's dtype."""
+    T = o.shape[0]
+    return (o.float().reshape(T, -1) * torch.sigmoid(g.float())).to(g.dtype)
+
+
+def relu_sq(z: torch.Tensor) -> torch.Tensor:
+    return torch.relu(z.float()).pow(2).to(z.dtype)
+
+
+def moe_route_sigmoid(scores: torch.Tensor, correction: torch.Tensor, k: int, scale: float):
+    """scores fp32 [T, >= E]: sigmoid router scores in the first E = len(correction)
+    columns.  The k experts with the largest score + correction (lowest index first among
+    equals); weights = their scores / (sum + 1e-20) * scale.  -> (fp32 [T, k], int32 [T, k])."""
+    E = correction.numel()
+    s = scores[:, :E].float()
+    ids = torch.topk(s + correction.float(), k, dim=-1).indices
+    w = torch.gather(s, 1, ids)
+    return w / (w.sum(-1, keepdim=True) + 1e-20) * scale, ids.to(torch.int32)
+
+
+def moe_finish(routed: Optional[torch.Tensor], dense: Optional[torch.Tensor],
+               topk_w: Optional[torch.Tensor], topk_ids: Optional[torch.Tensor],
+               shared: Optional[torch.Tensor], gate: Optional[torch.Tensor]) -> torch.Tensor:
+    """The routed experts' weighted sum -- ``routed`` [T, W] already combined, or gathered
+    from ``dense`` [E, T, W] (every expert's output for every token) with topk_w / topk_ids
+    -- plus gate[t] * shared[t] (gate fp32 [T], any stride)."""
+    if routed is not None:
+        out = routed.float()
+    else:
+        T = dense.shape[1]
+        y = dense.float()[topk_ids.long(), torch.arange(T, device=dense.device)[:, None]]
+        out = (y * topk_w.float()[:, :, None]).sum(1)
+    if shared is not None:
+        out = out + gate.float()[:, None] * shared.float()
+    return out.to(shared.dtype if shared is not None else (routed if routed is not None else dense).dtype)
+
+
+def side_gate(pre: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int) -> torch.Tensor:
+    """gelu_tanh(pre [T, n]) * table[ids, col0:col0 + n] in pre's dtype."""
+    n = pre.shape[1]
+    z = pre.float()
+    g = 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
+    return (g * table[ids.long(), col0:col0 + n].float()).to(pre.dtype)
