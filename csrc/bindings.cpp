@@ -23,6 +23,8 @@ int dt_code(const Tensor& t) {
   return -1;
 }
 
+bool act_dtype(const Tensor& t);
+
 hipStream_t stream() { return c10::hip::getCurrentHIPStreamMasqueradingAsCUDA().stream(); }
 
 void check_gpu(const Tensor& t, const char* name) {
@@ -78,8 +80,8 @@ void silu_mul(Tensor out, Tensor x) {
   c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
   TORCH_CHECK(x.dim() == 2 && x.is_contiguous() && out.is_contiguous(), "kgc.silu_mul: contiguous 2-D");
   const int64_t I = x.size(1) / 2;
-  TORCH_CHECK(x.size(1) % 16 == 0 && out.size(0) == x.size(0) && out.size(1) == I,
-              "kgc.silu_mul: shapes");
+  TORCH_CHECK(x.size(1) % 2 == 0 && out.size(0) == x.size(0) && out.size(1) == I &&
+              out.scalar_type() == x.scalar_type() && act_dtype(x), "kgc.silu_mul: shapes / dtypes");
   kgc::launch_silu_mul(dt_code(x), out.data_ptr(), x.data_ptr(), x.size(0), (int)I, stream());
 }
 
