@@ -103,7 +103,9 @@ def relu2_mlp(h, up, down):
     return np.maximum(h @ up.T, 0.0) ** 2 @ down.T
 
 
-def feed_forward(h, wts, L, mlp):
+def feed_forward(h, wts, L, mlp, margins=None):
+    """``margins`` (a list) receives, for a routed layer, each token's gap between the last
+    chosen and the first unchosen choice score: how close the routing decision was."""
     P = L + "mlp."
     if mlp["kind"] == "dense":
         return (silu(h @ wts[P + "gate"].T) * (h @ wts[P + "up"].T)) @ wts[P + "down"].T
@@ -111,6 +113,9 @@ def feed_forward(h, wts, L, mlp):
     s = sigmoid(h @ wts[P + "router"].T)
     choice = s + wts[P + "correction"]
     out = np.zeros_like(h)
+    if margins is not None and rt["top"] < rt["experts"]:
+        ranked = -np.sort(-choice, axis=-1)
+        margins.append(ranked[:, rt["top"] - 1] - ranked[:, rt["top"]])
     for t in range(h.shape[0]):
         top = np.argsort(-choice[t], kind="stable")[: rt["top"]]
         w = s[t, top] / (s[t, top].sum() + 1e-20) * rt["scale"]
@@ -142,8 +147,9 @@ def layer_runs(cfg):
     return runs + [(i, False) for i in range(b, n)]
 
 
-def forward(cfg, wts, tokens, taps=None):
-    """-> logits [n, vocab]; ``taps`` receives the residual stream after every layer run."""
+def forward(cfg, wts, tokens, taps=None, margins=None):
+    """-> logits [n, vocab]; ``taps`` receives the residual stream after every layer run,
+    ``margins`` the routing margins of every routed layer run (see feed_forward)."""
     tokens = np.asarray(tokens)
     eps, m = cfg["norm"]["eps"], cfg["residual_mult"]
     x = rms(wts["embed"][tokens], eps) * wts["embed.norm"]
@@ -159,7 +165,8 @@ def forward(cfg, wts, tokens, taps=None):
         else:
             x = x + m * latent_attention(h, wts, L, lay["mixer"], eps)
         if lay.get("mlp"):
-            x = x + m * feed_forward(rms(x, eps) * wts[L + "norm2"], wts, L, lay["mlp"])
+            x = x + m * feed_forward(rms(x, eps) * wts[L + "norm2"], wts, L, lay["mlp"],
+                                     margins)
         if side:
             x = x + m * side_input(x, tokens, wts, L, i, side["dim"], eps)
         if taps is not None:

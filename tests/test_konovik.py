@@ -1,0 +1,459 @@
+"""Konovik through the engine (registry, safetensors loading, block manager, state slots,
+step packing, kernels) against the plain numpy oracle in ``konovik_oracle.py``.
+
+Every test writes its own small config.json + model.safetensors (random bf16 weights)
+and drives the engine with the teacher-forced replayer or the generation entry points.
+CPU runs use the reference ops in fp32; ``-m gpu`` runs use the HIP kernels in fp32 and
+bf16.  Windows and pages are small (window 5..9, 8-token pages), so one key wrongly seen
+or missed, a lost state or a skipped pass changes the logits far beyond the tolerances."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import konovik_oracle as oracle
+from kubernetes_gpu_cluster_amd.engine.config import EngineConfig
+from kubernetes_gpu_cluster_amd.engine.llm_engine import LLM, LLMEngine
+from kubernetes_gpu_cluster_amd.engine.replay import TraceReplayer
+from kubernetes_gpu_cluster_amd.engine.sequence import SamplingParams
+
+CPU = pytest.param("cpu", "float32", id="cpu-fp32")
+GPU32 = pytest.param("cuda", "float32", marks=pytest.mark.gpu, id="gpu-fp32")
+GPU16 = pytest.param("cuda", "bfloat16", marks=pytest.mark.gpu, id="gpu-bf16")
+DEVICES = [CPU, GPU32, GPU16]
+# Row error: rms of the logit difference over the rms of the logits, means taken off.
+# fp32: every row within 3e-4.  bf16: rounding moves a row by a few percent (median within
+# 0.03, every row within 0.3) -- except where rounding flips a routing choice: a token whose
+# choice scores the oracle itself separates by less than MARGIN is a close call, and such a
+# row (and, through the recurrent state, the few after it) is only held to 2.0.  A key
+# wrongly seen or hidden, or a state lost, moves every later row by more than these.
+TOL = {"float32": 3e-4, "bfloat16": 0.3}
+TOL_MEDIAN = {"float32": 3e-4, "bfloat16": 0.03}
+MARGIN, AFTER = 0.03, 4
+
+
+def latent(heads=4, dim=12, rot=8, vdim=10, rank=24, size=7, scale=0.3, base=100.0,
+           scaling=(3.0, 16, 4.0, 1.0), mlp=None):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot, "vdim": vdim, "kv_rank": rank, "scale": scale}
+    if size:
+        m["mask"] = {"size": size}
+    if rot:
+        m["rot"] = {"dims": rot, "base": base}
+        if scaling:
+            f, o, fa, sl = scaling
+            m["rot"]["scaling"] = {"factor": f, "original": o, "fast": fa, "slow": sl}
+    return {"type": "latent_attention", "mixer": m, "mlp": mlp}
+
+
+def gru(width=40, mlp=None):
+    return {"type": "mingru", "mixer": {"width": width}, "mlp": mlp}
+
+
+def dense(ff=48):
+    return {"kind": "dense", "ff": ff}
+
+
+def moe(experts=6, top=2, ff=20, scale=1.3, shared=28):
+    m = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "scale": scale}}
+    if shared:
+        m["shared"] = {"ff": shared}
+    return m
+
+
+def config(layers, width=64, vocab=160, eps=1e-5, mult=0.4, loop=None, side=6):
+    c = {"architecture": "Konovik", "vocab": vocab, "width": width, "layers": layers,
+         "norm": {"eps": eps}, "residual_mult": mult}
+    if loop:
+        c["loop"] = dict(zip(("start", "stop", "times"), loop))
+    if side:
+        c["token_side"] = {"dim": side}
+    return c
+
+
+MIXED = config([latent(mlp=dense()), gru(mlp=moe()),
+                latent(heads=3, dim=8, rot=4, vdim=16, rank=20, size=5, scale=0.4, mlp=moe(shared=0)),
+                gru(width=24)], loop=(1, 3, 2))
+# values a model may make equal or 1, and parts it may leave out: one head, one expert used,
+# no loop, no side input, no frequency scaling, no window, rotary part as wide as the rest,
+# value size = key size, multiplier 1, a recurrent layer first and an attention layer last,
+# a loop of one pass
+PLAIN = config([gru(width=32, mlp=dense(32)),
+                latent(heads=1, dim=16, rot=16, vdim=16, rank=16, size=0, scaling=None,
+                       mlp=moe(experts=2, top=1, ff=16, scale=1.0, shared=0)),
+                latent(heads=2, dim=8, rot=2, vdim=8, rank=12, size=9, scaling=None)],
+               width=48, vocab=96, mult=1.0, loop=(0, 1, 1), side=0)
+# sizes the matrix-core prefill kernel, the 16-byte decode paths and the grouped expert GEMM
+# take (cache rows of 96 and 128 with values of 64 and 96, eight heads; experts of 128 on a
+# width of 128), windows over several key tiles, the whole stack looped three times
+WIDE = config([latent(heads=8, dim=32, rot=32, vdim=24, rank=64, size=40, scale=0.15,
+                      scaling=(4.0, 64, 8.0, 1.0), mlp=moe(experts=8, top=3, ff=128, shared=128)),
+               gru(width=96),
+               latent(heads=4, dim=16, rot=32, vdim=32, rank=96, size=70, scale=0.12, base=500.0,
+                      mlp=dense(96))],
+              width=128, vocab=200, mult=0.25, loop=(0, 3, 3), side=16)
+
+
+def write_model(path, cfg, seed):
+    """Random bf16 weights in the checkpoint's naming; returns them as float64 arrays."""
+    from safetensors.torch import save_file
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+    t = {}
+
+    def lin(name, out, inp, gain=1.0):
+        t[name] = torch.randn(out, inp, generator=g) * gain / inp ** 0.5
+
+    def vec(name, n, base, spread):
+        t[name] = base + spread * torch.randn(n, generator=g)
+
+    def one(name):
+        t[name] = torch.tensor(1.0 + 0.2 * float(torch.randn((), generator=g)))
+    t["embed"] = torch.randn(cfg["vocab"], W, generator=g)
+    one("embed.norm")
+    lin("head", cfg["vocab"], W, 2.0)
+    one("final.norm")
+    side = cfg.get("token_side")
+    if side:
+        t["side.embed"] = torch.randn(cfg["vocab"], len(cfg["layers"]) * side["dim"], generator=g)
+    for i, lc in enumerate(cfg["layers"]):
+        L, m = "l%d." % i, lc["mixer"]
+        one(L + "norm1")
+        t[L + "shift"] = torch.rand(W, generator=g)
+        if lc["type"] == "latent_attention":
+            H, d, r, dv, rank = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            lin(L + "mix.q", H * (d + r), W, 2.0)
+            lin(L + "mix.dkv", rank + r, W, 2.0)
+            vec(L + "mix.dkv.norm", rank, 1.0, 0.2)
+            lin(L + "mix.uk", H * d, rank, 2.0)
+            lin(L + "mix.uv", H * dv, rank)
+            lin(L + "mix.g", H * dv, W, 2.0)
+            lin(L + "mix.o", W, H * dv)
+        else:
+            n = m["width"]
+            lin(L + "mix.z", n, W, 2.0)
+            lin(L + "mix.x", n, W, 2.0)
+            lin(L + "mix.g", n, W, 2.0)
+            vec(L + "mix.z.b", n, 0.0, 1.0)
+            vec(L + "mix.x.b", n, 0.0, 0.5)
+            lin(L + "mix.o", W, n)
+        f = lc["mlp"]
+        if f:
+            one(L + "norm2")
+            if f["kind"] == "dense":
+                lin(L + "mlp.gate", f["ff"], W, 2.0)
+                lin(L + "mlp.up", f["ff"], W)
+                lin(L + "mlp.down", W, f["ff"])
+            else:
+                for e in range(f["router"]["experts"]):
+                    lin(L + "mlp.e%d.up" % e, f["expert"]["ff"], W, 2.0)
+                    lin(L + "mlp.e%d.down" % e, W, f["expert"]["ff"])
+                lin(L + "mlp.router", f["router"]["experts"], W, 3.0)
+                vec(L + "mlp.correction", f["router"]["experts"], 0.0, 0.3)
+                if f.get("shared"):
+                    lin(L + "mlp.shared.up", f["shared"]["ff"], W, 2.0)
+                    lin(L + "mlp.shared.down", W, f["shared"]["ff"])
+                    lin(L + "mlp.shared.sg", 1, W, 2.0)
+        if side:
+            lin(L + "side.gate", side["dim"], W, 2.0)
+            lin(L + "side.proj", W, side["dim"])
+            vec(L + "side.norm", W, 1.0, 0.2)
+    t = {k: v.to(torch.bfloat16).contiguous() for k, v in t.items()}
+    os.makedirs(path, exist_ok=True)
+    save_file(t, os.path.join(path, "model.safetensors"))
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    return {k: v.double().numpy() for k, v in t.items()}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    root = tmp_path_factory.mktemp("konovik")
+    out = {}
+    for name, cfg, seed in (("mixed", MIXED, 21), ("plain", PLAIN, 22), ("wide", WIDE, 23)):
+        d = str(root / name)
+        out[name] = (d, cfg, write_model(d, cfg, seed))
+    return out
+
+
+_engines = {}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _release_engines():
+    """Engines are shared by the tests of this module and released after the last one."""
+    yield
+    for eng in _engines.values():
+        eng.shutdown()
+    _engines.clear()
+    import gc
+    gc.collect()
+    if torch.cuda.is_available():
+        torch.cuda.empty_cache()
+
+
+def engine(models, name, device, dtype, pages=24, page=8, seqs=4, **kw):
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    key = (name, device, dtype, pages, page, seqs, tuple(sorted(kw.items())))
+    if key not in _engines:
+        d = models[name][0]
+        _engines[key] = LLMEngine(EngineConfig(
+            model=d, dtype=dtype, device=device, block_size=page, max_num_seqs=seqs,
+            max_model_len=pages * page, max_num_batched_tokens=pages * page,
+            num_gpu_blocks_override=pages + 1, cuda_graph_max_bs=seqs, **kw))
+    return _engines[key]
+
+
+def row_errs(got, want):
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    w = want - want.mean(-1, keepdims=True)
+    return np.sqrt((d ** 2).mean(-1) / (w ** 2).mean(-1))
+
+
+class Verdict:
+    def __init__(self, ok, text):
+        self.ok, self.text = ok, text
+
+    def __bool__(self):
+        return self.ok
+
+    def __repr__(self):
+        return self.text
+
+
+def expected(cfg, wts, toks):
+    """The oracle's logits, with the rows marked whose routing was a close call."""
+    margins = []
+    lg = oracle.forward(cfg, wts, toks, margins=margins)
+    shaky = np.zeros(len(toks), dtype=bool)
+    if margins:
+        for t in np.where(np.min(np.stack(margins), axis=0) < MARGIN)[0]:
+            shaky[t:t + 1 + AFTER] = True
+    return Expected(lg, shaky)
+
+
+class Expected:
+    def __init__(self, logits, shaky):
+        self.logits, self.shaky = logits, shaky
+
+    def __getitem__(self, key):
+        return Expected(self.logits[key], self.shaky[key])
+
+
+def close(got, want, dtype):
+    e = row_errs(got, want.logits)
+    firm = ~want.shaky if dtype != "float32" else np.ones(len(e), dtype=bool)
+    text = "rows %d (%d firm): median %.2g, worst firm %.2g, worst %.2g" % (
+        len(e), firm.sum(), np.median(e), e[firm].max() if firm.any() else 0.0, e.max())
+    ok = e.max() < (TOL[dtype] if dtype == "float32" else 2.0)
+    ok = ok and (not firm.any() or e[firm].max() < TOL[dtype])
+    if len(e) >= 8:
+        ok = ok and np.median(e) < TOL_MEDIAN[dtype]
+    return Verdict(bool(ok), text)
+
+
+def tokens_for(cfg, n, seed):
+    return np.random.default_rng(seed).integers(0, cfg["vocab"], n).tolist()
+
+
+def run_alone(rp, rid, toks, cuts):
+    """Feed `toks` in portions of the sizes `cuts` (the last size repeats); all logits."""
+    out, lo, i = [], 0, 0
+    while lo < len(toks):
+        n = cuts[min(i, len(cuts) - 1)]
+        i += 1
+        hi = min(len(toks), lo + n)
+        lg = rp.step([{"id": rid, "tokens": toks[lo:hi], "want": list(range(hi - lo))}],
+                     [rid] if hi == len(toks) else [])
+        out.append(lg.cpu().numpy())
+        lo = hi
+    return np.concatenate(out)
+
+
+# ---------------------------------------------------------------- whole prompts, decode, portions
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "plain", "wide"])
+def test_whole_prompt_matches_oracle(models, name, device, dtype):
+    _, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 150 if name == "wide" else 61, 1)
+    want = expected(cfg, wts, toks)
+    got = run_alone(rp, "w", toks, [len(toks)])
+    assert close(got, want, dtype)
+    # the first tokens of a sequence, and a one-token prompt
+    assert close(got[:3], want[:3], dtype)
+    one = run_alone(rp, "o", toks[:1], [1])
+    assert close(one, want[:1], dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "plain", "wide"])
+def test_prefill_then_token_by_token(models, name, device, dtype):
+    _, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 130 if name == "wide" else 70, 2)
+    want = expected(cfg, wts, toks)
+    if name == "wide":                             # portions across 64-row blocks and key tiles
+        assert close(run_alone(rp, "c", toks, [70, 3, 45, 2, 1]), want, dtype)
+    got = run_alone(rp, "d", toks, [20, 1])        # decoded tokens: every window passes
+    assert close(got, want, dtype)
+    got = run_alone(rp, "e", toks, [1])            # decoding from the very first token
+    assert close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("cuts", [[2], [3, 2, 7, 2, 11, 5, 1], [8], [9, 16, 2, 1]])
+def test_portions(models, device, dtype, cuts):
+    _, cfg, wts = models["mixed"]
+    eng = engine(models, "mixed", device, dtype)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 45, 3)
+    want = expected(cfg, wts, toks)
+    assert close(run_alone(rp, "p", toks, cuts), want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_long_decode(models, device, dtype):
+    _, cfg, wts = models["plain"]
+    eng = engine(models, "plain", device, dtype, pages=40)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 150, 4)
+    want = expected(cfg, wts, toks)
+    got = run_alone(rp, "l", toks, [5, 1])
+    assert close(got[-20:], want[-20:], dtype)
+    assert close(got, want, dtype)
+
+
+# ---------------------------------------------------------------- batches, pages and slots reused
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "wide"])
+def test_mixed_batches_and_reuse(models, name, device, dtype):
+    """Four live requests of unequal length, portions beside decode rows, requests that
+    sit out steps; the pool (14 pages) and the four slots are used again by later
+    requests.  Every row must match the request run alone (the oracle)."""
+    _, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype, pages=14)
+    rp = TraceReplayer(eng)
+    lens = {"a": 30, "b": 9, "c": 41, "d": 2, "e": 25, "f": 17, "g": 33}
+    toks = {k: tokens_for(cfg, n, 10 + i) for i, (k, n) in enumerate(lens.items())}
+    want = {k: expected(cfg, wts, v) for k, v in toks.items()}
+    at = {k: 0 for k in lens}
+    got = {k: [] for k in lens}
+    # (request, tokens) per step; a request is freed when its tokens are used up
+    plan = [[("a", 7), ("b", 3)], [("a", 1), ("b", 1), ("c", 12)], [("a", 1), ("c", 2), ("d", 2)],
+            [("b", 5), ("c", 1), ("a", 9)], [("a", 1), ("c", 1)], [("a", 11), ("c", 25), ("e", 4)],
+            [("e", 1), ("f", 17)], [("e", 1), ("g", 8)], [("e", 19), ("g", 1)], [("g", 24)]]
+    used_pages = []
+    for step in plan:
+        entries, end = [], []
+        for k, n in step:
+            lo = at[k]
+            entries.append({"id": k, "tokens": toks[k][lo:lo + n], "want": list(range(n))})
+            at[k] += n
+            if at[k] == lens[k]:
+                end.append(k)
+        assert len(rp.seqs) <= 4
+        lg = rp.step(entries, end).cpu().numpy()
+        for s in rp.seqs.values():
+            used_pages += s.block_ids
+        o = 0
+        for k, n in step:
+            got[k].append(lg[o:o + n])
+            o += n
+    assert all(at[k] == lens[k] for k in lens)
+    assert len(used_pages) > len(set(used_pages)) and len(set(used_pages)) <= 14
+    for k in lens:
+        assert close(np.concatenate(got[k]), want[k], dtype), k
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_slot_reuse_starts_from_zero_state(models, device, dtype):
+    """A slot that held a long request is given to a new one: its shift rows, recurrent
+    state and pages must not leak into the new request's first tokens."""
+    _, cfg, wts = models["mixed"]
+    eng = engine(models, "mixed", device, dtype, seqs=1, pages=10)
+    rp = TraceReplayer(eng)
+    first, second = tokens_for(cfg, 50, 20), tokens_for(cfg, 12, 21)
+    run_alone(rp, "x", first, [50])
+    got = run_alone(rp, "y", second, [4, 1])
+    assert close(got, expected(cfg, wts, second), dtype)
+
+
+# ---------------------------------------------------------------- residual stream per layer run
+@pytest.mark.parametrize("device,dtype", DEVICES)
+@pytest.mark.parametrize("name", ["mixed", "plain"])
+def test_layer_taps(models, name, device, dtype):
+    d, cfg, wts = models[name]
+    eng = engine(models, name, device, dtype)
+    runner = eng.executor.runner
+    toks = tokens_for(cfg, 19, 5)
+    want = []
+    oracle.forward(cfg, wts, toks, want)
+    assert len(want) == len(oracle.layer_runs(cfg))
+    rp = TraceReplayer(eng)
+    taps = []
+    model = runner.model
+    orig = model.forward
+    model.forward = lambda *a, **k: orig(*a, taps=taps, **k)
+    try:
+        run_alone(rp, "t", toks, [len(toks)])
+    finally:
+        model.forward = orig
+    assert len(taps) == len(want)
+    tol = 2e-4 if dtype == "float32" else 0.05
+    for got, w in zip(taps, want):
+        g = got.cpu().double().numpy()
+        assert np.abs(g - w).max() <= tol * np.abs(w).max()
+
+
+# ---------------------------------------------------------------- generation entry points
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_greedy_generation_through_scheduler(models, device, dtype):
+    """LLM.generate (request intake, continuous batching, chunked prefill with a token
+    budget smaller than the prompts, sampling at temperature 0): every generated token is
+    the oracle's argmax given the tokens before it."""
+    d, cfg, wts = models["mixed"]
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    llm = LLM(model=d, dtype=dtype, device=device, block_size=8, max_num_seqs=3,
+              max_model_len=96, max_num_batched_tokens=16, num_gpu_blocks_override=40,
+              cuda_graph_max_bs=3)
+    try:
+        prompts = [tokens_for(cfg, n, 30 + n) for n in (5, 23, 1, 37, 12)]
+        outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True))
+    finally:
+        llm.shutdown()
+    margin = 1e-3 if dtype == "float32" else 0.15
+    for p, o in zip(prompts, outs):
+        gen = list(o.output_token_ids)
+        assert len(gen) == 12
+        lg = oracle.forward(cfg, wts, p + gen)
+        for i, tok in enumerate(gen):
+            row = lg[len(p) - 1 + i]
+            assert row[tok] >= row.max() - margin * (row.max() - row.min()), (i, tok)
+
+
+def test_registry_and_config_reader(models):
+    from kubernetes_gpu_cluster_amd.models import resolve_model
+    d, cfg, _ = models["mixed"]
+    mc, wdir = resolve_model(d)
+    assert mc.arch == "konovik" and wdir == d and mc.num_layers == 4
+    assert [s.kind for s in mc.layer_specs] == ["latent_attention", "mingru", "latent_attention",
+                                                "mingru"]
+    assert [i for i, _ in mc.layer_runs()] == [0, 1, 2, 1, 2, 3]
+    assert [again for _, again in mc.layer_runs()] == [False, False, False, True, False, False]
+    sp = mc.layer_specs[2]
+    assert (sp.heads, sp.dim, sp.rot_dims, sp.vdim, sp.kv_rank) == (3, 8, 4, 16, 20)
+    assert sp.window.size == 5 and sp.rotary.interleaved and sp.rotary.yarn == (3.0, 16.0, 4.0, 1.0)
+    assert (sp.mlp.kind, sp.mlp.experts, sp.mlp.top, sp.mlp.shared_ff) == ("moe", 6, 2, 0)
+    assert mc.layer_specs[1].mlp.shared_ff == 28 and mc.layer_specs[3].mlp is None
+    assert mc.has_recurrent_state and mc.residual_mult == 0.4 and mc.side_dim == 6
+    mp, _ = resolve_model(models["plain"][0])
+    assert mp.layer_specs[1].window is None and mp.layer_specs[1].rotary.yarn is None
+    assert mp.side_dim == 0 and [i for i, _ in mp.layer_runs()] == [0, 1, 2]
