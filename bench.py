@@ -89,9 +89,10 @@ def parse():
     ap.add_argument("--log-level", default="WARNING",
                     help="python logging level on stderr (INFO shows the GEMM tuner's choices)")
     ap.add_argument("--compare-sizes", default="w2048,w4096",
-                    help="--mode compare: size suffixes of the dilavik-* / llama-* preset pairs")
+                    help="--mode compare: size suffixes of the <family>-<size> presets")
     ap.add_argument("--compare-families", default="dilavik,llama",
-                    help="--mode compare: which preset of each pair to run (profiling one alone)")
+                    help="--mode compare: the preset families to run at each size (dilavik, konovik, "
+                         "llama); ratios are taken against the last one")
     ap.add_argument("--mode", default="service", choices=["service", "engine", "compare"],
                     help="service: HTTP/SSE through API server + router (headline); "
                          "engine: LLMEngine.step() in-process")
@@ -642,7 +643,7 @@ def _compare_one(model: str, args) -> dict:
 
 
 def main_compare(args):
-    """--mode compare: the hybrid presets beside the Llama-style decoders of equal size
+    """--mode compare: the hybrid presets (dilavik, konovik) beside the Llama-style decoders of equal size
     (models/configs.py), same requests, same engine settings, one JSON line per model and a
     closing line with the ratios.  Random weights, synthetic prompts."""
     assert torch.cuda.is_available(), "bench.py --mode compare needs a GPU"
@@ -655,12 +656,12 @@ def main_compare(args):
                      dtype=args.dtype)
             print(json.dumps(r), flush=True)
             pair[fam] = r
-        if len(pair) == 2:
-            rows.append({"size": size,
-                         "prefill_ratio": round(pair["dilavik"]["prefill_tok_s"] /
-                                                pair["llama"]["prefill_tok_s"], 3),
-                         "decode_ratio": round(pair["dilavik"]["decode_tok_s"] /
-                                               pair["llama"]["decode_tok_s"], 3)})
+        fams = list(pair)
+        for fam in fams[:-1]:
+            base = pair[fams[-1]]
+            rows.append({"size": size, "model": fam, "against": fams[-1],
+                         "prefill_ratio": round(pair[fam]["prefill_tok_s"] / base["prefill_tok_s"], 3),
+                         "decode_ratio": round(pair[fam]["decode_tok_s"] / base["decode_tok_s"], 3)})
     print(json.dumps({"mode": "compare", "data": "synthetic", "weights": "random", "ratios": rows}))
 
 

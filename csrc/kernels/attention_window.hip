@@ -697,7 +697,10 @@ static void decode_dispatch(T* out, const T* q, const T* kc, const T* vc, const 
                             int dv, int krs, int vrs, int bs, int num_blocks, float scale, int window,
                             int keep_first, const float* gate, hipStream_t s) {
   const int qpg = H / G;
-  const int QH = qpg >= 8 ? 8 : qpg >= 3 ? 4 : qpg;      // heads per workgroup: 1, 2, 4, 8
+  int QH = qpg >= 8 ? 8 : qpg >= 3 ? 4 : qpg;            // heads per workgroup: 1, 2, 4, 8
+  // many heads on one key/value group and few rows: smaller head groups, so that the grid
+  // still covers the CUs (the groups re-read the rows from L2)
+  while (QH > 2 && (int64_t)D * G * ((qpg + QH - 1) / QH) < 256) QH >>= 1;
   const dim3 grid(D, G, (qpg + QH - 1) / QH);
   // 8 waves split a row's keys finest (shortest chain per workgroup); once the grid holds
   // two workgroups per CU, 4-wave workgroups let two of them overlap on a CU instead

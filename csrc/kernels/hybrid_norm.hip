@@ -272,15 +272,67 @@ void launch_gate_proj(int dtype, float* out, const void* h, const void* w, const
 namespace {
 
 // x += mult * a, a = add or add / rms(add) * anw; then out = x / rms(x) * w (w null: x;
-// out null: none).  out may be x itself (O = float).  A thread touches the same columns
-// in every pass, so it re-reads only what it wrote.
-template <typename T, typename O>
+// out null: none).  out may be x itself (O = float).  A thread owns columns threadIdx.x +
+// k NT; with EPT > 0 (W <= EPT * NT) it keeps them in registers, so x and add are read once
+// and x written once; EPT = 0 walks the row in passes, re-reading only what it wrote.
+template <typename T, typename O, int EPT>
 __global__ __launch_bounds__(NT) void residual_norm_kernel(
     O* out, float* x, const T* __restrict__ add, const float* __restrict__ anw,
     const float* __restrict__ w, float mult, int W, float eps) {
   __shared__ float scratch[NT / 64];
   const int64_t row = blockIdx.x;
   float* xr = x + row * W;
+  if constexpr (EPT > 0) {
+    float xv[EPT];
+#pragma unroll
+    for (int k = 0; k < EPT; ++k) {
+      const int c = threadIdx.x + k * NT;
+      xv[k] = c < W ? xr[c] : 0.f;
+    }
+    if (add != nullptr) {
+      const T* ar = add + row * W;
+      float av[EPT];
+#pragma unroll
+      for (int k = 0; k < EPT; ++k) {
+        const int c = threadIdx.x + k * NT;
+        av[k] = c < W ? to_f(ar[c]) : 0.f;
+      }
+      if (anw != nullptr) {
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < EPT; ++k) ss += av[k] * av[k];
+        ss = block_sum<NT>(ss, scratch);
+        const float ra = 1.f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+        for (int k = 0; k < EPT; ++k) {
+          const int c = threadIdx.x + k * NT;
+          if (c < W) av[k] = av[k] * ra * anw[c];
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < EPT; ++k) {
+        const int c = threadIdx.x + k * NT;
+        xv[k] += mult * av[k];
+        if (c < W) xr[c] = xv[k];
+      }
+    }
+    if (out == nullptr) return;
+    O* o = out + row * W;
+    float r = 1.f;
+    if (w != nullptr) {
+      float ss = 0.f;
+#pragma unroll
+      for (int k = 0; k < EPT; ++k) ss += xv[k] * xv[k];
+      ss = block_sum<NT>(ss, scratch);
+      r = 1.f / sqrtf(ss / (float)W + eps);
+    }
+#pragma unroll
+    for (int k = 0; k < EPT; ++k) {
+      const int c = threadIdx.x + k * NT;
+      if (c < W) o[c] = from_f<O>(w != nullptr ? xv[k] * r * w[c] : xv[k]);
+    }
+    return;
+  }
   if (add != nullptr) {
     const T* ar = add + row * W;
     if (anw != nullptr) {
@@ -354,13 +406,23 @@ void launch_residual_norm(int dtype, int out_dtype, void* out, float* x, const v
                           const float* anw, const float* w, float mult, int rows, int W,
                           float eps, hipStream_t s) {
   if (rows <= 0) return;
+#define KGC_RN(O, EPT)                                                          \
+  residual_norm_kernel<T, O, EPT><<<rows, NT, 0, s>>>((O*)out, x, (const T*)add, anw, w, mult, \
+                                                      W, eps)
+#define KGC_RN_W(O)                      \
+  do {                                   \
+    if (W <= 4 * NT) KGC_RN(O, 4);       \
+    else if (W <= 8 * NT) KGC_RN(O, 8);  \
+    else if (W <= 16 * NT) KGC_RN(O, 16); \
+    else KGC_RN(O, 0);                   \
+  } while (0)
   if (out == nullptr || out_dtype == DT_F32) {
-    KGC_DISPATCH_T(dtype, residual_norm_kernel<T, float><<<rows, NT, 0, s>>>(
-        (float*)out, x, (const T*)add, anw, w, mult, W, eps));
+    KGC_DISPATCH_T(dtype, KGC_RN_W(float));
   } else {
-    KGC_DISPATCH_T(dtype, residual_norm_kernel<T, T><<<rows, NT, 0, s>>>(
-        (T*)out, x, (const T*)add, anw, w, mult, W, eps));
+    KGC_DISPATCH_T(dtype, KGC_RN_W(T));
   }
+#undef KGC_RN_W
+#undef KGC_RN
 }
 
 void launch_gate_mul(int dtype, void* out, const void* o, int64_t st, int64_t sh, const void* g,

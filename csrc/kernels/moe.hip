@@ -629,15 +629,16 @@ namespace {
 // wins among equals); weights = the chosen scores / (their sum + 1e-20) * scale.
 constexpr int RS_MAX_PER_LANE = 16;          // E <= 1024
 
+template <int RS_PER_LANE>                   // experts per lane: E <= 64 * RS_PER_LANE
 __global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(
     float* __restrict__ w, int* __restrict__ ids, const float* __restrict__ scores,
     int64_t stride, const float* __restrict__ corr, int ntok, int E, int k, float scale) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (t >= ntok) return;
   const float* sr = scores + (int64_t)t * stride;
-  float sc[RS_MAX_PER_LANE], ch[RS_MAX_PER_LANE];
+  float sc[RS_PER_LANE], ch[RS_PER_LANE];
 #pragma unroll
-  for (int u = 0; u < RS_MAX_PER_LANE; ++u) {
+  for (int u = 0; u < RS_PER_LANE; ++u) {
     const int e = lane + 64 * u;
     sc[u] = e < E ? sr[e] : 0.f;
     ch[u] = e < E ? sc[u] + corr[e] : -INFINITY;
@@ -648,7 +649,7 @@ __global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(
     float best = -INFINITY, bs = 0.f;
     int bi = 0x7fffffff;
 #pragma unroll
-    for (int u = 0; u < RS_MAX_PER_LANE; ++u) {
+    for (int u = 0; u < RS_PER_LANE; ++u) {
       if (ch[u] > best) {               // strict: the lowest index of a lane's equals
         best = ch[u];
         bi = lane + 64 * u;
@@ -666,7 +667,7 @@ __global__ __launch_bounds__(256) void moe_route_sigmoid_kernel(
       }
     }
 #pragma unroll
-    for (int u = 0; u < RS_MAX_PER_LANE; ++u)
+    for (int u = 0; u < RS_PER_LANE; ++u)
       if (lane + 64 * u == bi) ch[u] = -INFINITY;
     sum += bs;
     if (j == lane) {                    // host checks k <= 64
@@ -713,8 +714,14 @@ void launch_moe_route_sigmoid(float* w, int* ids, const float* scores, int64_t s
                               const float* corr, int ntok, int E, int k, float scale,
                               hipStream_t s) {
   if (ntok <= 0) return;
-  moe_route_sigmoid_kernel<<<(ntok + 3) / 4, 256, 0, s>>>(w, ids, scores, stride, corr, ntok, E,
-                                                          k, scale);
+  const int grid = (ntok + 3) / 4;
+  if (E <= 64)
+    moe_route_sigmoid_kernel<1><<<grid, 256, 0, s>>>(w, ids, scores, stride, corr, ntok, E, k, scale);
+  else if (E <= 256)
+    moe_route_sigmoid_kernel<4><<<grid, 256, 0, s>>>(w, ids, scores, stride, corr, ntok, E, k, scale);
+  else
+    moe_route_sigmoid_kernel<RS_MAX_PER_LANE><<<grid, 256, 0, s>>>(w, ids, scores, stride, corr,
+                                                                   ntok, E, k, scale);
 }
 
 void launch_moe_finish(int dtype, void* out, const void* routed, const void* dense,

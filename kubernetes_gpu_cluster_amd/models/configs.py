@@ -321,6 +321,45 @@ PRESETS.update({
 })
 
 
+def _konovik(name: str, width: int, pattern: str, heads: int, gru_width: int, dense_ff: int,
+             expert_ff: int, shared_ff: int, loop: Optional[tuple], window: int = 1024,
+             vocab: int = 32000, rank: int = 192, dim: int = 128, rot: int = 64, vdim: int = 128,
+             experts: int = 8, top: int = 2, side: int = 64) -> ModelConfig:
+    """A Konovik-architecture preset: ``pattern`` is one letter per layer ("a": latent
+    attention, "g": minGRU); attention layers carry the gated dense feed-forward, minGRU
+    layers the routed experts (+ a shared one)."""
+    rs = RotarySpec(rot, 10000.0, interleaved=True, yarn=(4.0, 2048.0, 32.0, 1.0))
+    moe = FeedForwardSpec("moe", expert_ff, act="relu2", experts=experts, top=top,
+                          route_scale=1.5, shared_ff=shared_ff)
+    specs = tuple(
+        MixerSpec("latent_attention", heads, dim, vdim, kv_heads=1, scale=(dim + rot) ** -0.5,
+                  rot_dims=rot, window=WindowSpec(window), ff=dense_ff, kv_rank=rank, rotary=rs,
+                  mlp=FeedForwardSpec("dense", dense_ff))
+        if c == "a" else
+        MixerSpec("mingru", 1, gru_width, gru_width, ff=expert_ff, width=gru_width, mlp=moe)
+        for c in pattern)
+    return ModelConfig(name, "konovik", len(specs), width, heads, 1, dim, dense_ff, vocab,
+                       max_position=8192, rms_eps=1e-6, layer_specs=specs, residual_mult=0.3,
+                       layer_loop=loop, side_dim=side, token_shift=True, bos_token_id=1,
+                       eos_token_id=2)
+
+
+# Konovik presets beside the equal-width hybrid / Llama presets above: the same number of
+# layer runs (a looped pair counts twice), 16 / 32 heads, and a feed-forward whose ACTIVE
+# parameters per token (two of eight experts + the shared one, or the gated dense one) are
+# those of the Llama preset's; the cache row (192 + 64) is what the matrix-core prefill
+# kernel of the windowed attention covers.
+PRESETS.update({
+    "konovik-w2048": _konovik("konovik-w2048", 2048, "agagagagag", 16, 4096, 5504, 2048, 1536,
+                              (2, 4, 2)),
+    "konovik-w4096": _konovik("konovik-w4096", 4096, "agagag", 32, 8192, 14336, 4096, 4096,
+                              (2, 4, 2), window=2048),
+    "tiny-konovik": _konovik("tiny-konovik", 128, "agag", 4, 192, 256, 128, 128, (1, 3, 2),
+                             window=24, vocab=1024, rank=32, dim=16, rot=16, vdim=16, experts=4,
+                             side=16),
+})
+
+
 # HF repo basenames (lower-cased) -> preset
 _ALIASES = {
     "meta-llama-3-8b": "llama-3-8b", "meta-llama-3-8b-instruct": "llama-3-8b",

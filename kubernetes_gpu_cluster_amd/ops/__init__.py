@@ -897,7 +897,7 @@ def grouped_experts(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
     block_expert = torch.empty(rows // bm, dtype=torch.int32, device=dev)
     meta = torch.empty(1, dtype=torch.int32, device=dev)
     k.moe_align(sorted_ids, block_expert, meta, topk_ids.contiguous(), 0, E, bm)
-    inter = torch.zeros(rows, I, dtype=x.dtype, device=dev)
+    inter = torch.empty(rows, I, dtype=x.dtype, device=dev)
     k.moe_gemm(inter, x.contiguous(), w_up, sorted_ids, block_expert, meta, npairs, topk, bm,
                True, False)
     a = act(inter)

@@ -1,5 +1,5 @@
 """Microbenchmarks of the hybrid-decoder kernels beside the Llama-path kernel each one is
-closest to, at the layer shapes of the dilavik-w2048 / llama-w2048 presets.
+closest to, at the layer shapes of the dilavik-w2048 / konovik-w2048 / llama-w2048 presets.
 
     python tools/hybrid_bench.py [--reps 20] > profiles/hybrid_kernels.jsonl
 
@@ -174,11 +174,111 @@ def rows(reps):
              like="rope_kv_store")
 
 
+def konovik(reps):
+    """The Konovik-style kernels at the konovik-w2048 layer shapes, each beside the kernel of
+    the other hybrid decoder (or of the Llama / Mixtral path) it is closest to."""
+    # ---- latent attention: 16 heads over one cache row of 192 + 64 per token, window 1024
+    H, rank, r, bs, Wn = 16, 192, 64, 32, 1024
+    dk = rank + r
+    for name, P_q, P_sl, D_ctx in (("prefill 32x512", [512] * 32, [512] * 32, []),
+                                   ("prefill 8x2048", [2048] * 8, [2048] * 8, []),
+                                   ("decode 64 @544", [], [], [544] * 64),
+                                   ("decode 256 @544", [], [], [544] * 256)):
+        m, tables, nb = meta(P_q, P_sl, D_ctx, bs, DEV)
+        T = sum(P_q) + len(D_ctx)
+        q = torch.randn(T, H, dk, device=DEV, dtype=BF)
+        cache = torch.randn(nb, 1, bs, dk, device=DEV, dtype=BF)
+        pos = torch.zeros(T, dtype=torch.int64, device=DEV)
+        us = timed(lambda: ops.window_attention(q, cache, cache[..., :rank], pos, m, 0.07, Wn, 0,
+                                                None), reps)
+        pairs = sum(sum(min(p + 1, Wn) for p in range(sl - ql, sl)) for ql, sl in zip(P_q, P_sl))
+        if P_q:
+            emit("window_attention, latent rows (MFMA tile)", name, us,
+                 tflop=2 * pairs * (dk + rank) * H / 1e12, like="window_attention (MFMA tile)")
+        else:
+            emit("window_attention, latent rows (8-wave decode)", name, us,
+                 gbytes=sum(min(c, Wn) for c in D_ctx) * dk * 2 / 1e9,
+                 like="window_attention (8-wave decode)")
+    # ---- minGRU scan (width 4096) beside the mLSTM scan of the same rows
+    n_ch = 4096
+    for name, P_q, D_ctx in (("prefill 32x512", [512] * 32, []), ("prefill 2x8192", [8192] * 2, []),
+                             ("decode 64", [], [100] * 64), ("decode 256", [], [100] * 256)):
+        n = len(P_q) + len(D_ctx)
+        m, _, _ = meta(P_q, list(P_q), D_ctx, 32, DEV, slots=list(range(n)))
+        T = sum(P_q) + len(D_ctx)
+        zxg = torch.randn(T, 3 * n_ch, device=DEV, dtype=BF)
+        bias = torch.randn(2 * n_ch, device=DEV)
+        st = torch.zeros(n, n_ch, device=DEV)
+        us = timed(lambda: ops.mingru_scan(zxg, bias, st, m, n_ch, BF), reps)
+        emit("mingru_scan", name, us, gbytes=(T * n_ch * 8 + 2 * n * n_ch * 4) / 1e9, like="mlstm_scan")
+    W = 2048
+    for T in (16384, 64, 256):
+        x = torch.randn(T, W, device=DEV)
+        y = torch.randn(T, W, device=DEV, dtype=BF)
+        w = torch.ones(W, device=DEV)
+        us = timed(lambda: ops.residual_norm(x, y, 0.3, w, 1e-6, BF), reps)
+        emit("residual_norm (add, norm -> 16 bit)", f"{T}x{W}", us, gbytes=T * W * 12 / 1e9,
+             like="group_rms_norm(add)")
+        us = timed(lambda: ops.residual_norm(x, y, 0.3, w, 1e-6, torch.float32, add_norm_w=w), reps)
+        emit("residual_norm (normed add, norm -> fp32)", f"{T}x{W}", us, gbytes=T * W * 14 / 1e9,
+             like="group_rms_norm(add)")
+        n = 64 if T > 256 else T
+        P_q, D_ctx = ([T // n] * n, []) if T > 256 else ([], [100] * T)
+        m, _, _ = meta(P_q, list(P_q), D_ctx, 32, DEV, slots=list(range(n)))
+        h = torch.randn(T, W, device=DEV)
+        st = torch.zeros(n, W, device=DEV)
+        us = timed(lambda: ops.token_shift(h, w, st, m, BF), reps)
+        emit("token_shift", f"{T}x{W}", us, gbytes=T * W * (4 + 4 + 2) / 1e9, like="group_rms_norm(add)")
+        # latent cache rows + query rows beside rotary + store of the windowed attention
+        d = 128
+        proj = torch.randn(T, H * (d + r) + dk + H * d, device=DEV, dtype=BF)
+        q_lat = torch.randn(H, T, rank, device=DEV, dtype=BF)
+        nb = T // bs + 2
+        cache = torch.zeros(nb, 1, bs, dk, device=DEV, dtype=BF)
+        pos = (torch.arange(T, device=DEV) % 512).to(torch.int64)
+        slots = torch.arange(T, device=DEV, dtype=torch.int64) + bs
+        table = ref.rope_table_yarn(r, 4096, 1e4, (4.0, 2048.0, 32.0, 1.0)).to(DEV)
+        us = timed(lambda: ops.latent_rope_store(proj, q_lat, pos, table, torch.ones(rank, device=DEV),
+                                                 1e-6, cache, slots, H, d, r, rank), reps)
+        emit("latent_rope_store", f"{T} rows", us,
+             gbytes=T * (H * r * 2 + H * rank * 2 + H * dk * 2 + 2 * dk * 2) / 1e9, like="rope_kv_store")
+        o = torch.randn(H, T, d, device=DEV, dtype=BF)
+        g = torch.randn(T, H * d, device=DEV, dtype=BF)
+        us = timed(lambda: ops.gate_mul(o.transpose(0, 1), g), reps)
+        emit("gate_mul", f"{T}x{H * d}", us, gbytes=T * H * d * 6 / 1e9, like="head_norm_gate")
+        z = torch.randn(T * 2, 2048, device=DEV, dtype=BF)
+        us = timed(lambda: ops.relu_sq(z), reps)
+        emit("relu_sq", f"{2 * T}x2048", us, gbytes=T * 2 * 2048 * 4 / 1e9, like="silu_mul (K7)")
+        # routing: 8 experts + the shared gate, top 2
+        hb = torch.randn(T, W, device=DEV, dtype=BF)
+        wg = torch.randn(9, W, device=DEV, dtype=BF)
+        us = timed(lambda: ops.gate_proj(hb, wg, None, ops.GATE_SIGMOID), reps)
+        emit("gate_proj N=9 (router scores)", f"{T}x{W}", us, gbytes=T * W * 2 / 1e9, like="gate_proj N=16")
+        sc = torch.rand(T, 9, device=DEV)
+        corr = torch.randn(8, device=DEV) * 0.1
+        us = timed(lambda: ops.moe_route_sigmoid(sc, corr, 2, 1.5), reps)
+        emit("moe_route_sigmoid", f"{T}x8 top 2", us, gbytes=T * (36 + 16) / 1e9)
+        lg = torch.randn(T, 8, device=DEV, dtype=BF)
+        us = timed(lambda: ops.moe_topk_softmax(lg, 2), reps)
+        emit("moe_topk_softmax (K13)", f"{T}x8 top 2", us, gbytes=T * (16 + 16) / 1e9,
+             like="moe_route_sigmoid")
+        routed = torch.randn(T, W, device=DEV, dtype=BF)
+        shared = torch.randn(T, W, device=DEV, dtype=BF)
+        us = timed(lambda: ops.moe_finish(routed, None, None, None, shared, sc[:, 8]), reps)
+        emit("moe_finish (routed + gated shared)", f"{T}x{W}", us, gbytes=T * W * 6 / 1e9,
+             like="silu_mul (K7)")
+        pre = torch.randn(T, 64, device=DEV, dtype=BF)
+        ids = torch.randint(0, 32000, (T,), device=DEV)
+        tab = torch.randn(32000, 640, device=DEV, dtype=BF)
+        us = timed(lambda: ops.side_gate(pre, ids, tab, 128), reps)
+        emit("side_gate", f"{T}x64", us, gbytes=T * 64 * 6 / 1e9)
+
+
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--reps", type=int, default=20)
-    ap.add_argument("--only", default="attention,recurrent,rows")
+    ap.add_argument("--only", default="attention,recurrent,rows,konovik")
     a = ap.parse_args()
     ops.load_extension(strict=True)
     for part in a.only.split(","):
-        {"attention": attention, "recurrent": recurrent, "rows": rows}[part](a.reps)
+        {"attention": attention, "recurrent": recurrent, "rows": rows, "konovik": konovik}[part](a.reps)
