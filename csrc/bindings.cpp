@@ -1564,7 +1564,7 @@ void token_shift(Tensor out, Tensor h, Tensor mu, Tensor state, std::optional<Te
 
 void mingru_scan(Tensor out, Tensor zxg, Tensor bias, Tensor state, std::optional<Tensor> qsl,
                  std::optional<Tensor> seq_lens, std::optional<Tensor> ctx_lens, Tensor slots,
-                 int64_t P, int64_t D, int64_t Tp, int64_t width) {
+                 int64_t P, int64_t D, int64_t Tp, int64_t width, bool blocked) {
   check_gpu(zxg, "zxg");
   check_f32(bias, "bias");
   check_f32(state, "state");
@@ -1578,10 +1578,13 @@ void mingru_scan(Tensor out, Tensor zxg, Tensor bias, Tensor state, std::optiona
   TORCH_CHECK(bias.numel() == 2 * width && state.dim() == 2 && state.size(1) == width,
               "kgc.mingru_scan: bias [2 width], state [slots, width]");
   const StepSeqs q = step_seqs(qsl, seq_lens, ctx_lens, slots, P, D, Tp, T);
+  const int nblk = blocked ? kgc::mingru_scan_blocks((int)P, (int)Tp, (int)width) : 0;
+  Tensor ws;
+  if (nblk > 0) ws = at::empty({nblk, 2, width}, state.options());
   kgc::launch_mingru_scan(dt_code(zxg), out.data_ptr(), zxg.data_ptr(), zxg.stride(0),
                           bias.data_ptr<float>(), state.data_ptr<float>(), q.qsl, q.sl, q.ctx,
                           q.slots, (int)P, (int)D, (int)Tp, (int)width, (int)state.size(0),
-                          stream());
+                          nblk > 0 ? ws.data_ptr<float>() : nullptr, nblk, stream());
 }
 
 void latent_rope_store(Tensor q_out, Tensor proj, Tensor q_lat, Tensor positions,
@@ -1738,7 +1741,7 @@ TORCH_LIBRARY(kgc, m) {
   m.def("token_shift(Tensor(a!) out, Tensor h, Tensor mu, Tensor(b!) state, Tensor? qsl, Tensor? seq_lens, "
         "Tensor? ctx_lens, Tensor slots, int P, int D, int Tp) -> ()");
   m.def("mingru_scan(Tensor(a!) out, Tensor zxg, Tensor bias, Tensor(b!) state, Tensor? qsl, "
-        "Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int width) -> ()");
+        "Tensor? seq_lens, Tensor? ctx_lens, Tensor slots, int P, int D, int Tp, int width, bool blocked=True) -> ()");
   m.def("latent_rope_store(Tensor(a!) q_out, Tensor proj, Tensor q_lat, Tensor positions, Tensor? table, "
         "Tensor norm_w, float eps, Tensor(b!) cache, Tensor slots, int H, int d, int r, int rank) -> ()");
   m.def("gate_mul(Tensor(a!) out, Tensor o, Tensor g) -> ()");

@@ -63,7 +63,7 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(
   }
 }
 
-constexpr int MAX_DV_PER_LANE = 8;     // dv <= 512
+constexpr int MAX_DV_PER_LANE = 16;    // dv <= 1024
 
 // grid (T, H), one wave.  LDS: q row [dk] fp32, p [64], value-row offsets [64].
 template <typename T>

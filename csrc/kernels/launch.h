@@ -314,7 +314,10 @@ void launch_token_shift(int out_dtype, void* out, const float* h, const float* m
 void launch_mingru_scan(int dtype, void* out, const void* zxg, int64_t stride, const float* bias,
                         float* state, const int* qsl, const int* seq_lens, const int* ctx_lens,
                         const int* slots, int P, int D, int Tp, int width, int num_slots,
-                        hipStream_t s);
+                        float* ws, int ws_blocks, hipStream_t s);
+// blocks of the block-parallel prefill path for this step (0: token-order scan), each
+// needing 2 * width floats of workspace
+int mingru_scan_blocks(int P, int Tp, int width);
 void launch_latent_rope_store(int dtype, void* q_out, const void* proj, int64_t proj_stride,
                               const void* q_lat, const int64_t* positions, const float* table,
                               int table_rows, const float* nw, float eps, void* cache,

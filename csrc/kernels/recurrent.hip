@@ -309,8 +309,8 @@ __global__ __launch_bounds__(64) void mingru_scan_kernel(
     T* __restrict__ out, const T* __restrict__ zxg, int64_t stride,
     const float* __restrict__ bias, float* __restrict__ state, const int* __restrict__ qsl,
     const int* __restrict__ seq_lens, const int* __restrict__ ctx_lens,
-    const int* __restrict__ slots, int P, int Tp, int width, int num_slots) {
-  const int s = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+    const int* __restrict__ slots, int P, int Tp, int width, int num_slots, int s0) {
+  const int s = blockIdx.x + s0, c = blockIdx.y * 64 + threadIdx.x;
   if (c >= width) return;
   int start, len, pos0;
   if (s < P) {
@@ -355,7 +355,137 @@ __global__ __launch_bounds__(64) void mingru_scan_kernel(
   *st = S;
 }
 
+// Long prefill chunks of few sequences: the chunk is cut into blocks of MG_BLOCK tokens that
+// run in parallel.  S_t = a_t S_(t-1) + b_t composes: a block maps its incoming state S to
+// A S + B with A = prod a_t and B its own scan from zero.
+//   reduce  every block's (A, B) per channel                       -> ws[block][0 / 1]
+//   carry   per sequence, in block order: ws[block][0] = incoming S; S = A S + B
+//   apply   every block again, in token order from its incoming S: the outputs, and the
+//           last block stores the sequence's state
+// A block's incoming state differs from the token-by-token value by rounding only.
+constexpr int MG_BLOCK = 64;
+
+struct BlockOfSeq { int seq, lb, nb; };
+
+// block b of the step -> its sequence, its index in it, the sequence's block count
+__device__ __forceinline__ BlockOfSeq block_of_seq(int b, const int* qsl, int P) {
+  BlockOfSeq r{-1, 0, 0};
+  int acc = 0;
+  for (int i = 0; i < P; ++i) {
+    const int nb = (qsl[i + 1] - qsl[i] + MG_BLOCK - 1) / MG_BLOCK;
+    if (b < acc + nb) {
+      r.seq = i;
+      r.lb = b - acc;
+      r.nb = nb;
+      return r;
+    }
+    acc += nb;
+  }
+  return r;
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void mingru_block_reduce_kernel(
+    float* __restrict__ ws, const T* __restrict__ zxg, int64_t stride,
+    const float* __restrict__ bias, const int* __restrict__ qsl, int P, int width) {
+  const int c = blockIdx.y * 64 + threadIdx.x;
+  const BlockOfSeq bq = block_of_seq(blockIdx.x, qsl, P);
+  if (c >= width || bq.seq < 0) return;
+  const int start = qsl[bq.seq] + bq.lb * MG_BLOCK;
+  const int len = min(MG_BLOCK, qsl[bq.seq + 1] - start);
+  const float bz = bias[c], bx = bias[width + c];
+  float A = 1.f, B = 0.f;
+  for (int t0 = 0; t0 < len; t0 += MG_UNROLL) {
+    float zv[MG_UNROLL], uv[MG_UNROLL];
+#pragma unroll
+    for (int u = 0; u < MG_UNROLL; ++u) {
+      const T* row = zxg + (int64_t)(start + min(t0 + u, len - 1)) * stride;
+      zv[u] = to_f(row[c]);
+      uv[u] = to_f(row[width + c]);
+    }
+#pragma unroll
+    for (int u = 0; u < MG_UNROLL; ++u) {
+      if (t0 + u < len) {
+        const float z = sigmoidf_(zv[u] + bz);
+        const float x = uv[u] + bx;
+        const float cand = x >= 0.f ? x + 0.5f : sigmoidf_(x);
+        A *= 1.f - z;
+        B = (1.f - z) * B + z * cand;
+      }
+    }
+  }
+  ws[((int64_t)blockIdx.x * 2 + 0) * width + c] = A;
+  ws[((int64_t)blockIdx.x * 2 + 1) * width + c] = B;
+}
+
+__global__ __launch_bounds__(64) void mingru_block_carry_kernel(
+    float* __restrict__ ws, const float* __restrict__ state, const int* __restrict__ qsl,
+    const int* __restrict__ seq_lens, const int* __restrict__ slots, int width, int num_slots) {
+  const int s = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+  if (c >= width) return;
+  int base = 0;
+  for (int i = 0; i < s; ++i) base += (qsl[i + 1] - qsl[i] + MG_BLOCK - 1) / MG_BLOCK;
+  const int len = qsl[s + 1] - qsl[s];
+  const int nb = (len + MG_BLOCK - 1) / MG_BLOCK;
+  const int slot = slots[s];
+  const bool fresh = seq_lens[s] - len <= 0 || slot < 0 || slot >= num_slots;
+  float S = fresh ? 0.f : state[(int64_t)slot * width + c];
+  for (int b = base; b < base + nb; ++b) {
+    float* w0 = ws + ((int64_t)b * 2 + 0) * width + c;
+    const float A = *w0, B = w0[width];
+    *w0 = S;
+    S = A * S + B;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(64) void mingru_block_apply_kernel(
+    T* __restrict__ out, const float* __restrict__ ws, const T* __restrict__ zxg, int64_t stride,
+    const float* __restrict__ bias, float* __restrict__ state, const int* __restrict__ qsl,
+    const int* __restrict__ slots, int P, int width, int num_slots) {
+  const int c = blockIdx.y * 64 + threadIdx.x;
+  const BlockOfSeq bq = block_of_seq(blockIdx.x, qsl, P);
+  if (c >= width || bq.seq < 0) return;
+  const int start = qsl[bq.seq] + bq.lb * MG_BLOCK;
+  const int len = min(MG_BLOCK, qsl[bq.seq + 1] - start);
+  const int slot = slots[bq.seq];
+  if (slot < 0 || slot >= num_slots) {                 // a padding sequence
+    for (int t = start; t < start + len; ++t) out[(int64_t)t * width + c] = from_f<T>(0.f);
+    return;
+  }
+  const float bz = bias[c], bx = bias[width + c];
+  float S = ws[((int64_t)blockIdx.x * 2) * width + c];
+  for (int t0 = 0; t0 < len; t0 += MG_UNROLL) {
+    float zv[MG_UNROLL], uv[MG_UNROLL], gv[MG_UNROLL];
+#pragma unroll
+    for (int u = 0; u < MG_UNROLL; ++u) {
+      const T* row = zxg + (int64_t)(start + min(t0 + u, len - 1)) * stride;
+      zv[u] = to_f(row[c]);
+      uv[u] = to_f(row[width + c]);
+      gv[u] = to_f(row[2 * width + c]);
+    }
+#pragma unroll
+    for (int u = 0; u < MG_UNROLL; ++u) {
+      if (t0 + u < len) {
+        const float z = sigmoidf_(zv[u] + bz);
+        const float x = uv[u] + bx;
+        const float cand = x >= 0.f ? x + 0.5f : sigmoidf_(x);
+        S = (1.f - z) * S + z * cand;
+        const float g = gv[u];
+        out[(int64_t)(start + t0 + u) * width + c] = from_f<T>(S * (g * sigmoidf_(g)));
+      }
+    }
+  }
+  if (bq.lb == bq.nb - 1) state[(int64_t)slot * width + c] = S;
+}
+
 }  // namespace
+
+int mingru_scan_blocks(int P, int Tp, int width) {
+  // blocks pay off when the sequences alone leave most CUs idle and the chunks are long
+  const bool on = P > 0 && Tp / P >= 8 * MG_BLOCK && (int64_t)P * ((width + 63) / 64) < 1024;
+  return on ? Tp / MG_BLOCK + P : 0;
+}
 
 void launch_token_shift(int out_dtype, void* out, const float* h, const float* mu, float* state,
                         const int* qsl, const int* seq_lens, const int* ctx_lens,
@@ -376,21 +506,32 @@ void launch_token_shift(int out_dtype, void* out, const float* h, const float* m
 void launch_mingru_scan(int dtype, void* out, const void* zxg, int64_t stride, const float* bias,
                         float* state, const int* qsl, const int* seq_lens, const int* ctx_lens,
                         const int* slots, int P, int D, int Tp, int width, int num_slots,
-                        hipStream_t s) {
+                        float* ws, int ws_blocks, hipStream_t s) {
   if (P + D <= 0) return;
-  const dim3 grid(P + D, (width + 63) / 64);
-  if (dtype == DT_BF16)
-    mingru_scan_kernel<bf16><<<grid, 64, 0, s>>>((bf16*)out, (const bf16*)zxg, stride, bias, state,
-                                                 qsl, seq_lens, ctx_lens, slots, P, Tp, width,
-                                                 num_slots);
-  else if (dtype == DT_F16)
-    mingru_scan_kernel<f16><<<grid, 64, 0, s>>>((f16*)out, (const f16*)zxg, stride, bias, state,
-                                                qsl, seq_lens, ctx_lens, slots, P, Tp, width,
-                                                num_slots);
-  else
-    mingru_scan_kernel<float><<<grid, 64, 0, s>>>((float*)out, (const float*)zxg, stride, bias,
-                                                  state, qsl, seq_lens, ctx_lens, slots, P, Tp,
-                                                  width, num_slots);
+  const int cg = (width + 63) / 64;
+  int s0 = 0, ns = P + D;
+#define KGC_MG(T)                                                                               \
+  do {                                                                                          \
+    if (ws != nullptr && ws_blocks > 0) {                                                       \
+      const dim3 gb(ws_blocks, cg);                                                             \
+      mingru_block_reduce_kernel<T><<<gb, 64, 0, s>>>(ws, (const T*)zxg, stride, bias, qsl, P,  \
+                                                      width);                                   \
+      mingru_block_carry_kernel<<<dim3(P, cg), 64, 0, s>>>(ws, state, qsl, seq_lens, slots,     \
+                                                           width, num_slots);                   \
+      mingru_block_apply_kernel<T><<<gb, 64, 0, s>>>((T*)out, ws, (const T*)zxg, stride, bias,  \
+                                                     state, qsl, slots, P, width, num_slots);   \
+      s0 = P;                                                                                   \
+      ns = D;                                                                                   \
+    }                                                                                           \
+    if (ns > 0)                                                                                 \
+      mingru_scan_kernel<T><<<dim3(ns, cg), 64, 0, s>>>((T*)out, (const T*)zxg, stride, bias,   \
+                                                        state, qsl, seq_lens, ctx_lens, slots,  \
+                                                        P, Tp, width, num_slots, s0);           \
+  } while (0)
+  if (dtype == DT_BF16) KGC_MG(bf16);
+  else if (dtype == DT_F16) KGC_MG(f16);
+  else KGC_MG(float);
+#undef KGC_MG
 }
 
 }  // namespace kgc

@@ -824,13 +824,15 @@ def mingru_scan(zxg: torch.Tensor, bias: torch.Tensor, state: torch.Tensor, meta
                 out_dtype: torch.dtype) -> torch.Tensor:
     """The minGRU recurrence over every step sequence's rows from / into state
     [slots, width] fp32, times silu of the output-gate columns: zxg [T, 3 width] holds the
-    update-gate | candidate | output-gate pre-activations, bias fp32 [2 width]."""
+    update-gate | candidate | output-gate pre-activations, bias fp32 [2 width].  Long chunks
+    of few sequences run block-parallel (KGC_MINGRU_SCAN=token keeps the token-order scan)."""
     if not _gpu(zxg):
         return ref.mingru_scan(zxg, bias, state, ref.step_sequences(meta), width, out_dtype)
     out = torch.empty(zxg.shape[0], width, dtype=out_dtype, device=zxg.device)
     _k().mingru_scan(out, zxg, bias, state, meta.query_start_loc, meta.prefill_seq_lens,
                      meta.decode_ctx_lens, meta.state_slots, meta.num_prefills,
-                     meta.num_decodes, meta.num_prefill_tokens, width)
+                     meta.num_decodes, meta.num_prefill_tokens, width,
+                     os.environ.get("KGC_MINGRU_SCAN", "block") != "token")
     return out
 
 

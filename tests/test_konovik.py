@@ -93,6 +93,13 @@ WIDE = config([latent(heads=8, dim=32, rot=32, vdim=24, rank=64, size=40, scale=
                latent(heads=4, dim=16, rot=32, vdim=32, rank=96, size=70, scale=0.12, base=500.0,
                       mlp=dense(96))],
               width=128, vocab=200, mult=0.25, loop=(0, 3, 3), side=16)
+# sizes that are multiples of nothing: odd vocabulary and width, cache rows whose bytes are no
+# multiple of 16, five experts, a window of one token, one layer looped three times
+ODD = config([gru(width=50, mlp=moe(experts=5, top=2, ff=18, scale=0.8, shared=10)),
+              latent(heads=3, dim=10, rot=6, vdim=14, rank=21, size=1, scale=0.35, base=30.0,
+                     scaling=(2.0, 8, 2.0, 0.5), mlp=dense(26)),
+              latent(heads=5, dim=6, rot=2, vdim=4, rank=9, size=11, scale=0.5, scaling=None)],
+             width=70, vocab=251, eps=1e-6, mult=0.7, loop=(2, 3, 3), side=5)
 
 
 def write_model(path, cfg, seed):
@@ -171,7 +178,8 @@ def write_model(path, cfg, seed):
 def models(tmp_path_factory):
     root = tmp_path_factory.mktemp("konovik")
     out = {}
-    for name, cfg, seed in (("mixed", MIXED, 21), ("plain", PLAIN, 22), ("wide", WIDE, 23)):
+    for name, cfg, seed in (("mixed", MIXED, 21), ("plain", PLAIN, 22), ("wide", WIDE, 23),
+                            ("odd", ODD, 24)):
         d = str(root / name)
         out[name] = (d, cfg, write_model(d, cfg, seed))
     return out
@@ -276,7 +284,7 @@ def run_alone(rp, rid, toks, cuts):
 
 # ---------------------------------------------------------------- whole prompts, decode, portions
 @pytest.mark.parametrize("device,dtype", DEVICES)
-@pytest.mark.parametrize("name", ["mixed", "plain", "wide"])
+@pytest.mark.parametrize("name", ["mixed", "plain", "wide", "odd"])
 def test_whole_prompt_matches_oracle(models, name, device, dtype):
     _, cfg, wts = models[name]
     eng = engine(models, name, device, dtype)
@@ -292,7 +300,7 @@ def test_whole_prompt_matches_oracle(models, name, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", DEVICES)
-@pytest.mark.parametrize("name", ["mixed", "plain", "wide"])
+@pytest.mark.parametrize("name", ["mixed", "plain", "wide", "odd"])
 def test_prefill_then_token_by_token(models, name, device, dtype):
     _, cfg, wts = models[name]
     eng = engine(models, name, device, dtype)
@@ -327,6 +335,20 @@ def test_long_decode(models, device, dtype):
     want = expected(cfg, wts, toks)
     got = run_alone(rp, "l", toks, [5, 1])
     assert close(got[-20:], want[-20:], dtype)
+    assert close(got, want, dtype)
+
+
+@pytest.mark.parametrize("device,dtype", DEVICES)
+def test_long_prompt(models, device, dtype):
+    """A prompt of several hundred tokens in one step (the recurrent layer's block-parallel
+    prefill on the GPU), then a second portion and decoded tokens that continue its state."""
+    _, cfg, wts = models["plain"]
+    eng = engine(models, "plain", device, dtype, pages=100)
+    rp = TraceReplayer(eng)
+    toks = tokens_for(cfg, 760, 6)
+    want = expected(cfg, wts, toks)
+    got = run_alone(rp, "L", toks, [600, 130, 1])
+    assert close(got[-40:], want[-40:], dtype)
     assert close(got, want, dtype)
 
 

@@ -169,6 +169,15 @@ def test_mingru_alone(dev, cuts):
     np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
 
 
+@pytest.mark.parametrize("dev", DEV)
+def test_mingru_long_chunks(dev):
+    """Chunks long enough for the block-parallel scan (blocks of 64 tokens, a ragged last
+    block), continued from and handing over to the token-order scan."""
+    dev = dev_of(dev)
+    got, want = _mingru_case(dev, 70, 24, 1300, [3, 650, 1, 1, 577, 20, 1], 11)
+    np.testing.assert_allclose(got, want, rtol=3e-4, atol=3e-4)
+
+
 # ---------------------------------------------------------------- latent attention
 def _latent_case(dev, spec, hidden, h, cuts, page, seed, eps=1e-5, prepare=None):
     """Run the LatentAttention module over a sequence cut into steps -> ([n, hidden], oracle)."""
