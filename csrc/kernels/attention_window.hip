@@ -266,7 +266,9 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
   float* pw = pb + wave * QH * 64;
   int* ow = ob + wave * 64;
   const int lpr = dv >> 3;                 // lanes per value row in the 16-byte path
-  const bool vrow = (dv & 7) == 0 && lpr <= 64 && (lpr & (lpr - 1)) == 0;
+  const bool vrow = (dv & 7) == 0 && lpr >= 1 && lpr <= 64;
+  const bool vpow2 = (lpr & (lpr - 1)) == 0;
+  const int kg = vrow ? 64 / lpr : 1;      // lane groups (lanes past kg * lpr idle)
   for (int chunk = wave; chunk < nchunks; chunk += NWV) {
     const int idx = chunk * 64 + lane;
     const bool ok = idx < total;
@@ -328,9 +330,9 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
       for (int h = 0; h < QH; ++h)
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[h][e >> 1][e & 1] *= alpha[h];
-      const int ci = lane & (lpr - 1), cg = lane / lpr, kg = 64 / lpr;
+      const int cg = lane / lpr, ci = lane - cg * lpr;
       constexpr int VB = std::is_same_v<T, float> ? 4 : 8;    // rows in flight per lane
-      for (int j0 = cg; j0 < cnt; j0 += VB * kg) {
+      for (int j0 = cg < kg ? cg : cnt; j0 < cnt; j0 += VB * kg) {
         Raw8<T> raw[VB];
 #pragma unroll
         for (int b = 0; b < VB; ++b) {
@@ -397,13 +399,25 @@ __global__ __launch_bounds__(64 * NWV) void window_decode_kernel(
     for (int w = 0; w < NWV; ++w) M = fmaxf(M, mm[w * QH + h]);
     f[h] = m[h] == -INFINITY ? 0.f : expf(m[h] - M);
   }
-  if (vrow) {
+  if (vrow && vpow2) {
     for (int off = lpr; off < 64; off <<= 1)
 #pragma unroll
       for (int h = 0; h < QH; ++h)
 #pragma unroll
         for (int e = 0; e < 8; ++e)
           acc[h][e >> 1][e & 1] += __shfl_xor(acc[h][e >> 1][e & 1], off, 64);
+  } else if (vrow) {
+    // lane groups of any width: the first group gathers the others' sums (lanes past it
+    // read wrapped lanes; their sums are not used)
+#pragma unroll
+    for (int h = 0; h < QH; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float own = acc[h][e >> 1][e & 1];
+        float tot = own;
+        for (int g2 = 1; g2 < kg; ++g2) tot += __shfl(own, (lane + g2 * lpr) & 63, 64);
+        acc[h][e >> 1][e & 1] = tot;
+      }
   }
   for (int w = 0; w < NWV; ++w) {
     if (vrow) {
