@@ -328,9 +328,9 @@ def _konovik(name: str, width: int, pattern: str, heads: int, gru_width: int, de
     """A Konovik-architecture preset: ``pattern`` is one letter per layer ("a": latent
     attention, "g": minGRU); attention layers carry the gated dense feed-forward, minGRU
     layers the routed experts (+ a shared one)."""
-    rs = RotarySpec(rot, 10000.0, interleaved=True, yarn=(4.0, 2048.0, 32.0, 1.0))
+    rs = RotarySpec(rot, 10000.0, interleaved=True, yarn=(8.0, 4096.0, 16.0, 2.0))
     moe = FeedForwardSpec("moe", expert_ff, act="relu2", experts=experts, top=top,
-                          route_scale=1.5, shared_ff=shared_ff)
+                          route_scale=2.5, shared_ff=shared_ff)
     specs = tuple(
         MixerSpec("latent_attention", heads, dim, vdim, kv_heads=1, scale=(dim + rot) ** -0.5,
                   rot_dims=rot, window=WindowSpec(window), ff=dense_ff, kv_rank=rank, rotary=rs,
@@ -339,7 +339,7 @@ def _konovik(name: str, width: int, pattern: str, heads: int, gru_width: int, de
         MixerSpec("mingru", 1, gru_width, gru_width, ff=expert_ff, width=gru_width, mlp=moe)
         for c in pattern)
     return ModelConfig(name, "konovik", len(specs), width, heads, 1, dim, dense_ff, vocab,
-                       max_position=8192, rms_eps=1e-6, layer_specs=specs, residual_mult=0.3,
+                       max_position=8192, rms_eps=1e-6, layer_specs=specs, residual_mult=0.5,
                        layer_loop=loop, side_dim=side, token_shift=True, bos_token_id=1,
                        eos_token_id=2)
 

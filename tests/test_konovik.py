@@ -461,6 +461,29 @@ def test_greedy_generation_through_scheduler(models, device, dtype):
             assert row[tok] >= row.max() - margin * (row.max() - row.min()), (i, tok)
 
 
+@pytest.mark.parametrize("device,dtype", [CPU, GPU16])
+def test_preset_with_random_weights_generates(device, dtype):
+    """The built-in small preset with random weights through request intake, the scheduler
+    and sampling (temperature > 0, top-k): the right number of tokens, all in range, and
+    the same tokens again for the same seeds."""
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    outs = []
+    for _ in range(2):
+        llm = LLM(model="tiny-konovik", dtype=dtype, device=device, random_init=True, seed=3,
+                  block_size=16, max_num_seqs=4, max_model_len=128, max_num_batched_tokens=64,
+                  num_gpu_blocks_override=40, cuda_graph_max_bs=4)
+        try:
+            prompts = [list(range(5, 5 + n)) for n in (3, 40, 17)]
+            res = llm.generate(prompts, SamplingParams(temperature=0.8, top_k=20, max_tokens=9,
+                                                       ignore_eos=True, seed=11))
+        finally:
+            llm.shutdown()
+        outs.append([list(o.output_token_ids) for o in res])
+    assert all(len(o) == 9 and all(0 <= t < 1024 for t in o) for o in outs[0])
+    assert outs[0] == outs[1]
+
+
 def test_registry_and_config_reader(models):
     from kubernetes_gpu_cluster_amd.models import resolve_model
     d, cfg, _ = models["mixed"]

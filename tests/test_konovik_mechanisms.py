@@ -120,7 +120,7 @@ def test_token_shift_over_steps(dev, cuts):
 @pytest.mark.parametrize("dev", DEV)
 def test_yarn_table_and_side_gate(dev):
     dev = dev_of(dev)
-    for dims, base, yarn in ((8, 100.0, (3.0, 16.0, 4.0, 1.0)), (32, 20000.0, (4.0, 2048.0, 32.0, 1.0)),
+    for dims, base, yarn in ((8, 100.0, (3.0, 16.0, 4.0, 1.0)), (16, 5000.0, (8.0, 1024.0, 16.0, 2.0)),
                              (6, 50.0, None)):
         sc = dict(zip(("factor", "original", "fast", "slow"), yarn)) if yarn else None
         f, mag = oracle.yarn_frequencies(dims, base, sc)

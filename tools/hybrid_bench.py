@@ -237,7 +237,7 @@ def konovik(reps):
         cache = torch.zeros(nb, 1, bs, dk, device=DEV, dtype=BF)
         pos = (torch.arange(T, device=DEV) % 512).to(torch.int64)
         slots = torch.arange(T, device=DEV, dtype=torch.int64) + bs
-        table = ref.rope_table_yarn(r, 4096, 1e4, (4.0, 2048.0, 32.0, 1.0)).to(DEV)
+        table = ref.rope_table_yarn(r, 4096, 1e4, (8.0, 4096.0, 16.0, 2.0)).to(DEV)
         us = timed(lambda: ops.latent_rope_store(proj, q_lat, pos, table, torch.ones(rank, device=DEV),
                                                  1e-6, cache, slots, H, d, r, rank), reps)
         emit("latent_rope_store", f"{T} rows", us,
