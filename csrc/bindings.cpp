@@ -1669,6 +1669,48 @@ void side_gate(Tensor out, Tensor pre, Tensor ids, Tensor table, int64_t col0) {
                         (int)n, stream());
 }
 
+bool side_input_rows(std::optional<Tensor> out, Tensor x, std::optional<Tensor> y, Tensor wg,
+                     Tensor wp, Tensor ids, Tensor table, int64_t col0, Tensor side_w,
+                     std::optional<Tensor> w, double mult, double eps) {
+  check_f32(x, "x");
+  check_f32(side_w, "side_w");
+  c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+  TORCH_CHECK(x.dim() == 2 && wg.dim() == 2 && wp.dim() == 2, "kgc.side_input_rows: shapes");
+  const int64_t T = x.size(0), W = x.size(1), n = wg.size(0);
+  if (!wg.is_cuda() || !kgc::side_input_rows_ok(dt_code(wg), (int)T, (int)W, (int)n)) return false;
+  auto same = [&](const Tensor& t) {
+    return t.is_cuda() && t.scalar_type() == wg.scalar_type() && t.device() == x.device();
+  };
+  TORCH_CHECK(wg.is_contiguous() && wg.size(1) == W && same(wp) && wp.is_contiguous() &&
+              wp.size(0) == W && wp.size(1) == n && wg.device() == x.device(),
+              "kgc.side_input_rows: gate [n, W], proj [W, n]");
+  TORCH_CHECK(same(table) && table.dim() == 2 && table.stride(1) == 1 && col0 >= 0 &&
+              col0 + n <= table.size(1), "kgc.side_input_rows: table [vocab, >= col0 + n]");
+  TORCH_CHECK(ids.is_cuda() && ids.scalar_type() == at::kLong && ids.numel() == T &&
+              ids.is_contiguous(), "kgc.side_input_rows: ids int64 [T]");
+  TORCH_CHECK(side_w.numel() == W, "kgc.side_input_rows: side_w [W]");
+  const void* yp = nullptr;
+  if (y.has_value()) {
+    TORCH_CHECK(same(*y) && y->is_contiguous() && y->sizes() == x.sizes(), "kgc.side_input_rows: y");
+    yp = y->data_ptr();
+  }
+  void* op = nullptr;
+  int odt = kgc::DT_F32;
+  if (out.has_value()) {
+    TORCH_CHECK(out->is_cuda() && out->is_contiguous() && out->sizes() == x.sizes() &&
+                out->device() == x.device() && w.has_value(), "kgc.side_input_rows: out with its weight");
+    odt = dt_code(*out);
+    TORCH_CHECK(odt == kgc::DT_F32 || odt == dt_code(wg), "kgc.side_input_rows: out dtype");
+    op = out->data_ptr();
+  }
+  kgc::launch_side_input_rows(dt_code(wg), odt, op, x.data_ptr<float>(), yp, wg.data_ptr(),
+                              wp.data_ptr(), ids.data_ptr<int64_t>(), table.data_ptr(),
+                              table.stride(0), (int)table.size(0), (int)col0,
+                              side_w.data_ptr<float>(), f32_opt(w, W, "w"), (float)mult, (int)T,
+                              (int)W, (int)n, (float)eps, stream());
+  return true;
+}
+
 void moe_route_sigmoid(Tensor w, Tensor ids, Tensor scores, Tensor correction, double scale) {
   check_f32(w, "w");
   check_f32(correction, "correction");
@@ -1747,6 +1789,8 @@ TORCH_LIBRARY(kgc, m) {
   m.def("gate_mul(Tensor(a!) out, Tensor o, Tensor g) -> ()");
   m.def("relu_sq(Tensor(a!) out, Tensor z) -> ()");
   m.def("side_gate(Tensor(a!) out, Tensor pre, Tensor ids, Tensor table, int col0) -> ()");
+  m.def("side_input_rows(Tensor(a!)? out, Tensor(b!) x, Tensor? y, Tensor wg, Tensor wp, Tensor ids, "
+        "Tensor table, int col0, Tensor side_w, Tensor? w, float mult, float eps) -> bool");
   m.def("moe_route_sigmoid(Tensor(a!) w, Tensor(b!) ids, Tensor scores, Tensor correction, float scale) -> ()");
   m.def("moe_finish(Tensor(a!) out, Tensor? routed, Tensor? dense, Tensor? topk_w, Tensor? topk_ids, "
         "Tensor? shared, Tensor? gate) -> ()");
@@ -1888,6 +1932,7 @@ TORCH_LIBRARY_IMPL(kgc, CUDA, m) {
   m.impl("gate_mul", &gate_mul);
   m.impl("relu_sq", &relu_sq);
   m.impl("side_gate", &side_gate);
+  m.impl("side_input_rows", &side_input_rows);
   m.impl("moe_route_sigmoid", &moe_route_sigmoid);
   m.impl("moe_finish", &moe_finish);
   m.impl("rms_norm", &rms_norm);

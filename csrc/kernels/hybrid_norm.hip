@@ -400,7 +400,147 @@ __global__ __launch_bounds__(NT) void side_gate_kernel(
   }
 }
 
+// The per-token side input of a layer for a few rows (decode steps), one workgroup per row:
+//   x += mult * y;  pre = W_g x;  g = gelu_tanh(pre) * table[id, col0 + :];  v = W_p g;
+//   x += mult * v / rms(v) * sw;  out = x / rms(x) * w  (w null: no output)
+// in one kernel instead of a cast, two small GEMMs, the gate and the add + norm.  Products
+// accumulate in fp32 and are rounded to T where the GEMM path rounds (its inputs and
+// outputs), so rows that take this kernel agree with rows that take the GEMMs to rounding
+// order.  16-bit T, W % 8 == 0, W <= EPT * 1024 threads, n % 8 == 0, n <= 512.
+constexpr int SI_NT = 1024, SI_JB = 4;
+
+template <typename T, typename O, int EPT>
+__global__ __launch_bounds__(SI_NT) void side_input_rows_kernel(
+    O* out, float* x, const T* __restrict__ y, const T* __restrict__ wg,
+    const T* __restrict__ wp, const int64_t* __restrict__ ids, const T* __restrict__ table,
+    int64_t ts, int vocab, int col0, const float* __restrict__ sw, const float* __restrict__ w,
+    float mult, int W, int n, float eps) {
+  extern __shared__ float lds[];
+  float* xb = lds;                 // [W]: x as the GEMM reads it (rounded to T)
+  float* gs = lds + W;             // [n]
+  __shared__ float scratch[SI_NT / 64];
+  const int64_t row = blockIdx.x;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float* xr = x + row * W;
+  float xv[EPT];
+#pragma unroll
+  for (int k = 0; k < EPT; ++k) {
+    const int c = threadIdx.x + k * SI_NT;
+    xv[k] = 0.f;
+    if (c < W) {
+      xv[k] = xr[c] + (y != nullptr ? mult * to_f(y[row * W + c]) : 0.f);
+      xb[c] = to_f(from_f<T>(xv[k]));
+    }
+  }
+  __syncthreads();
+  int64_t id = ids[row];
+  if (id < 0 || id >= vocab) id = 0;
+  const T* e = table + id * ts + col0;
+  const int chunks = W >> 3;
+  // a wave takes SI_JB outputs at a time, their weight rows' loads all in flight
+  constexpr int NWV = SI_NT / 64;
+  for (int j0 = wave * SI_JB; j0 < n; j0 += NWV * SI_JB) {
+    float acc[SI_JB];
+#pragma unroll
+    for (int b = 0; b < SI_JB; ++b) acc[b] = 0.f;
+    for (int ch = lane; ch < chunks; ch += 64) {
+      Pack8<T> p[SI_JB];
+#pragma unroll
+      for (int b = 0; b < SI_JB; ++b)
+        p[b].u = *reinterpret_cast<const u32x4*>(wg + (int64_t)min(j0 + b, n - 1) * W + 8 * ch);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) {
+        const float xq = xb[8 * ch + q];
+#pragma unroll
+        for (int b = 0; b < SI_JB; ++b) acc[b] += xq * to_f(p[b].h[q]);
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < SI_JB; ++b) {
+      const float tot = wave_sum(acc[b]);
+      const int j = j0 + b;
+      if (lane == 0 && j < n) {
+        const float z = to_f(from_f<T>(tot));
+        const float gl = 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+        gs[j] = to_f(from_f<T>(gl * to_f(e[j])));
+      }
+    }
+  }
+  __syncthreads();
+  float vv[EPT], ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < EPT; ++k) {
+    const int c = threadIdx.x + k * SI_NT;
+    vv[k] = 0.f;
+    if (c < W) {
+      const T* pr = wp + (int64_t)c * n;
+      float acc = 0.f;
+      for (int j0 = 0; j0 < n; j0 += 8) {
+        Pack8<T> p;
+        p.u = *reinterpret_cast<const u32x4*>(pr + j0);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) acc += gs[j0 + q] * to_f(p.h[q]);
+      }
+      vv[k] = to_f(from_f<T>(acc));
+      ss += vv[k] * vv[k];
+    }
+  }
+  ss = block_sum<SI_NT>(ss, scratch);
+  const float ra = 1.f / sqrtf(ss / (float)W + eps);
+  float s2 = 0.f;
+#pragma unroll
+  for (int k = 0; k < EPT; ++k) {
+    const int c = threadIdx.x + k * SI_NT;
+    if (c < W) {
+      xv[k] += mult * (vv[k] * ra * sw[c]);
+      xr[c] = xv[k];
+      s2 += xv[k] * xv[k];
+    }
+  }
+  if (out == nullptr || w == nullptr) return;
+  s2 = block_sum<SI_NT>(s2, scratch);
+  const float r = 1.f / sqrtf(s2 / (float)W + eps);
+  O* o = out + row * W;
+#pragma unroll
+  for (int k = 0; k < EPT; ++k) {
+    const int c = threadIdx.x + k * SI_NT;
+    if (c < W) o[c] = from_f<O>(xv[k] * r * w[c]);
+  }
+}
+
 }  // namespace
+
+bool side_input_rows_ok(int dtype, int rows, int W, int n) {
+  return (dtype == DT_BF16 || dtype == DT_F16) && rows <= 256 && W % 8 == 0 && W <= 4 * SI_NT &&
+         n % 8 == 0 && n <= 512;
+}
+
+void launch_side_input_rows(int dtype, int out_dtype, void* out, float* x, const void* y,
+                            const void* wg, const void* wp, const int64_t* ids,
+                            const void* table, int64_t ts, int vocab, int col0, const float* sw,
+                            const float* w, float mult, int rows, int W, int n, float eps,
+                            hipStream_t s) {
+  if (rows <= 0) return;
+  const size_t lds = (size_t)(W + n) * sizeof(float);
+#define KGC_SI(T, O, EPT)                                                                     \
+  side_input_rows_kernel<T, O, EPT><<<rows, SI_NT, lds, s>>>(                                  \
+      (O*)out, x, (const T*)y, (const T*)wg, (const T*)wp, ids, (const T*)table, ts, vocab,   \
+      col0, sw, w, mult, W, n, eps)
+#define KGC_SI_W(T, O)                     \
+  do {                                     \
+    if (W <= SI_NT) KGC_SI(T, O, 1);          \
+    else if (W <= 2 * SI_NT) KGC_SI(T, O, 2); \
+    else KGC_SI(T, O, 4);                     \
+  } while (0)
+  const bool f32out = out == nullptr || out_dtype == DT_F32;
+  if (dtype == DT_BF16) {
+    if (f32out) KGC_SI_W(bf16, float); else KGC_SI_W(bf16, bf16);
+  } else {
+    if (f32out) KGC_SI_W(f16, float); else KGC_SI_W(f16, f16);
+  }
+#undef KGC_SI_W
+#undef KGC_SI
+}
 
 void launch_residual_norm(int dtype, int out_dtype, void* out, float* x, const void* add,
                           const float* anw, const float* w, float mult, int rows, int W,

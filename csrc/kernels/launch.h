@@ -307,6 +307,12 @@ void launch_relu_sq(int dtype, void* out, const void* z, int64_t n, hipStream_t 
 void launch_side_gate(int dtype, void* out, const void* pre, const int64_t* ids,
                       const void* table, int64_t ts, int vocab, int col0, int rows, int n,
                       hipStream_t s);
+bool side_input_rows_ok(int dtype, int rows, int W, int n);
+void launch_side_input_rows(int dtype, int out_dtype, void* out, float* x, const void* y,
+                            const void* wg, const void* wp, const int64_t* ids,
+                            const void* table, int64_t ts, int vocab, int col0, const float* sw,
+                            const float* w, float mult, int rows, int W, int n, float eps,
+                            hipStream_t s);
 void launch_token_shift(int out_dtype, void* out, const float* h, const float* mu, float* state,
                         const int* qsl, const int* seq_lens, const int* ctx_lens,
                         const int* slots, int P, int Tp, int T, int W, int num_slots,

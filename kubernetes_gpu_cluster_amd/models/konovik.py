@@ -22,8 +22,9 @@ Kernel sequence per layer run (ops/__init__.py, "Konovik-style decoders"):
       latent_rope_store -> window_attention -> batched GEMM (values) -> gate_mul -> o GEMM
     minGRU: merged GEMM -> mingru_scan -> o GEMM
   -> residual_norm -> feed-forward (gate_up GEMM -> silu_mul -> down GEMM | gate_proj ->
-  moe_route_sigmoid -> expert GEMMs with relu_sq -> moe_finish) -> residual_norm (cast) ->
-  side gate GEMM -> side_gate -> side proj GEMM -> residual_norm (normed add + next norm).
+  moe_route_sigmoid -> expert GEMMs with relu_sq -> moe_finish) -> side_input (decode-size
+  batches: one kernel; otherwise residual_norm (cast) -> side gate GEMM -> side_gate -> side
+  proj GEMM -> residual_norm (normed add + next norm)).
 One GPU per replica (TP = PP = 1).
 """
 from __future__ import annotations
@@ -203,21 +204,19 @@ class KonovikForCausalLM(nn.Module):
             nxt = self.final_norm if last else self.layers[self.runs[n + 1][0]].norm1
             again = not last and self.runs[n + 1][3]
             out_dt = dt if last else f32
+            split = again or taps is not None       # the stream is needed before the next norm
             if layer.side_gate is not None:
-                xb = ops.residual_norm(x, y, m, None, eps, dt)
-                g = ops.side_gate(layer.side_gate(xb), input_ids, self.side_embed,
-                                  i * cfg.side_dim)
-                y, nw = layer.side_proj(g), layer.side_norm
+                h = ops.side_input(x, y, m, layer.side_gate.weight, layer.side_proj.weight,
+                                   input_ids, self.side_embed, i * cfg.side_dim, layer.side_norm,
+                                   None if split else nxt, eps, None if split else out_dt)
             else:
-                nw = None
-            if again or taps is not None:
-                ops.residual_norm(x, y, m, None, eps, None, add_norm_w=nw)
+                h = ops.residual_norm(x, y, m, None if split else nxt, eps,
+                                      None if split else out_dt)
+            if split:
                 if taps is not None:
                     taps.append(x.clone())
-                y, add_m, nw = (self.embed_out[:T], 1.0, None) if again else (None, 1.0, None)
-                h = ops.residual_norm(x, y, add_m, nxt, eps, out_dt)
-            else:
-                h = ops.residual_norm(x, y, m, nxt, eps, out_dt, add_norm_w=nw)
+                h = ops.residual_norm(x, self.embed_out[:T] if again else None, 1.0, nxt, eps,
+                                      out_dt)
         return h
 
     def compute_logits(self, hidden: torch.Tensor, gather: bool = True) -> torch.Tensor:

@@ -933,3 +933,26 @@ def side_gate(pre: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: i
     out = torch.empty_like(pre)
     _k().side_gate(out, pre.contiguous(), ids, table, col0)
     return out
+
+
+def side_input(x: torch.Tensor, y: Optional[torch.Tensor], mult: float, gate_w: torch.Tensor,
+               proj_w: torch.Tensor, ids: torch.Tensor, table: torch.Tensor, col0: int,
+               side_w: torch.Tensor, next_w: Optional[torch.Tensor], eps: float,
+               out_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
+    """The end of a layer with a per-token side input, on the fp32 stream x [T, W] in place:
+    x += mult * y (the feed-forward's output);  v = proj_w (gelu_tanh(gate_w x) *
+    table[ids, col0:col0 + n]);  x += mult * v / rms(v) * side_w;  returns x / rms(x) * next_w
+    in out_dtype (None: nothing).  Decode-size batches of 16-bit activations run as one
+    kernel; otherwise a cast, two GEMMs, ``side_gate`` and ``residual_norm``."""
+    from .gemm import linear
+    if _gpu(x) and x.shape[0] <= 256 and os.environ.get("KGC_SIDE_INPUT", "fused") != "gemm":
+        out = (torch.empty(x.shape, dtype=out_dtype, device=x.device)
+               if out_dtype is not None and next_w is not None else None)
+        if _k().side_input_rows(out, x, y, gate_w, proj_w, ids, table, col0, side_w,
+                                next_w if out is not None else None, float(mult), eps):
+            return out
+    xb = residual_norm(x, y, mult, None, eps, gate_w.dtype)
+    g = side_gate(linear(xb, gate_w), ids, table, col0)
+    if next_w is None:
+        out_dtype = None
+    return residual_norm(x, linear(g, proj_w), mult, next_w, eps, out_dtype, add_norm_w=side_w)

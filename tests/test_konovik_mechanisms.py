@@ -139,6 +139,38 @@ def test_yarn_table_and_side_gate(dev):
                                rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("dev,dtype", [pytest.param("cpu", torch.float32, id="cpu"),
+                                       pytest.param("cuda", torch.float32, marks=pytest.mark.gpu, id="gpu-fp32"),
+                                       pytest.param("cuda", torch.bfloat16, marks=pytest.mark.gpu, id="gpu-bf16")])
+@pytest.mark.parametrize("rows", [3, 300])
+def test_side_input_end_of_layer(dev, dtype, rows):
+    """x += m y; the gated side projection, RMS-normed, joins x; then the next norm.  Few
+    rows of 16-bit activations take the one-kernel path on the GPU, many rows the GEMMs."""
+    dev = dev_of(dev)
+    rng = np.random.default_rng(12)
+    W, n, vocab, layer = 72, 8, 40, 2
+    rnd = lambda *sh: torch.tensor(rng.normal(size=sh), dtype=torch.float32).to(dtype)   # noqa: E731
+    x = torch.tensor(rng.normal(size=(rows, W)) * 2, dtype=torch.float32)
+    y, wg, wp, table = rnd(rows, W), rnd(n, W) / 6, rnd(W, n), rnd(vocab, 4 * n)
+    sw, nw = rng.normal(size=W) + 1, rng.normal(size=W) + 1
+    ids = rng.integers(0, vocab, rows)
+    xs = x.clone().to(dev)
+    h = ops.side_input(xs, y.to(dev), 0.4, wg.to(dev), wp.to(dev), torch.tensor(ids, device=dev),
+                       table.to(dev), layer * n, f32(sw, dev), f32(nw, dev), 1e-5, torch.float32)
+    d = lambda t: t.float().double().numpy()   # noqa: E731
+    x1 = x.double().numpy() + 0.4 * d(y)
+    wts = {"side.embed": d(table), "side.gate": d(wg), "side.proj": d(wp), "side.norm": sw}
+    x2 = x1 + 0.4 * oracle.side_input(x1, ids, wts, "", layer, n, 1e-5)
+    tol = 3e-4 if dtype == torch.float32 else 4e-2
+    np.testing.assert_allclose(xs.cpu().numpy(), x2, rtol=tol, atol=tol)
+    np.testing.assert_allclose(h.cpu().numpy(), oracle.rms(x2, 1e-5) * nw, rtol=tol, atol=tol)
+    # without a next norm: the stream only
+    xs = x.clone().to(dev)
+    assert ops.side_input(xs, y.to(dev), 0.4, wg.to(dev), wp.to(dev), torch.tensor(ids, device=dev),
+                          table.to(dev), layer * n, f32(sw, dev), None, 1e-5, None) is None
+    np.testing.assert_allclose(xs.cpu().numpy(), x2, rtol=tol, atol=tol)
+
+
 # ---------------------------------------------------------------- minGRU
 def _mingru_case(dev, width, hidden, n, cuts, seed):
     get_state()

@@ -267,6 +267,19 @@ def konovik(reps):
         us = timed(lambda: ops.moe_finish(routed, None, None, None, shared, sc[:, 8]), reps)
         emit("moe_finish (routed + gated shared)", f"{T}x{W}", us, gbytes=T * W * 6 / 1e9,
              like="silu_mul (K7)")
+        if T <= 256:
+            import os
+            wsg = torch.randn(64, W, device=DEV, dtype=BF) / 45
+            wsp = torch.randn(W, 64, device=DEV, dtype=BF) / 8
+            tab2 = torch.randn(32000, 640, device=DEV, dtype=BF)
+            ids2 = torch.randint(0, 32000, (T,), device=DEV)
+            for mode in ("fused", "gemm"):
+                os.environ["KGC_SIDE_INPUT"] = mode
+                us = timed(lambda: ops.side_input(x, y, 0.3, wsg, wsp, ids2, tab2, 128, w, w, 1e-6,
+                                                  torch.float32), reps)
+                emit(f"side_input ({'one kernel' if mode == 'fused' else 'cast, 2 GEMMs, gate, add + norm'})",
+                     f"{T}x{W}", us)
+            os.environ.pop("KGC_SIDE_INPUT")
         pre = torch.randn(T, 64, device=DEV, dtype=BF)
         ids = torch.randint(0, 32000, (T,), device=DEV)
         tab = torch.randn(32000, 640, device=DEV, dtype=BF)
