@@ -210,6 +210,37 @@ def test_mingru_long_chunks(dev):
     np.testing.assert_allclose(got, want, rtol=3e-4, atol=3e-4)
 
 
+@pytest.mark.parametrize("dev", DEV)
+def test_mingru_scan_long_chunk_beside_decode_rows(dev):
+    """One step holds two long chunks (one from position 0, one continuing a state) and two
+    decode rows of other sequences; plain numpy recurrences are the expectation."""
+    dev = dev_of(dev)
+    rng = np.random.default_rng(13)
+    n, lens = 70, [700, 530]
+    T = sum(lens) + 2
+    zxg, bias = rng.normal(size=(T, 3 * n)), rng.normal(size=2 * n) * 0.5
+    state = rng.normal(size=(5, n))
+    m, _ = meta_for([(0, lens[0]), (40, lens[1])], [9, 0], None, dev, [3, 1, 0, 4])
+    st = f32(state, dev)
+    got = ops.mingru_scan(f32(zxg, dev), f32(bias, dev), st, m, n, torch.float32).cpu().numpy()
+    z = oracle.sigmoid(zxg[:, :n] + bias[:n])
+    u = zxg[:, n:2 * n] + bias[n:]
+    cand = np.where(u >= 0, u + 0.5, oracle.sigmoid(u))
+    gate = oracle.silu(zxg[:, 2 * n:])
+    want, end = np.zeros((T, n)), {}
+    for a, ln, s0, slot in ((0, 700, None, 3), (700, 530, state[1], 1), (1230, 1, state[0], 0),
+                            (1231, 1, None, 4)):
+        S = np.zeros(n) if s0 is None else s0.copy()
+        for t in range(a, a + ln):
+            S = (1 - z[t]) * S + z[t] * cand[t]
+            want[t] = S * gate[t]
+        end[slot] = S
+    np.testing.assert_allclose(got, want, rtol=3e-4, atol=3e-4)
+    for slot, S in end.items():
+        np.testing.assert_allclose(st[slot].cpu().numpy(), S, rtol=3e-4, atol=3e-4)
+    np.testing.assert_allclose(st[2].cpu().numpy(), state[2], rtol=1e-6)      # untouched
+
+
 # ---------------------------------------------------------------- latent attention
 def _latent_case(dev, spec, hidden, h, cuts, page, seed, eps=1e-5, prepare=None):
     """Run the LatentAttention module over a sequence cut into steps -> ([n, hidden], oracle)."""
